@@ -47,7 +47,10 @@ def resolve_architecture(cfg: dict) -> Architecture:
     (the reference's order, format/arch/base.py:91-123); an unknown name is an
     error that lists what is registered (format/arch/base.py:84-87).
     """
-    for name in cfg.get("architectures") or []:
+    named = list(cfg.get("architectures") or [])
+    if isinstance(cfg.get("architecture"), str):      # some configs name one architecture, not a list
+        named.append(cfg["architecture"])
+    for name in named:
         if name in ARCHITECTURES:
             return ARCHITECTURES[name]
     mt = cfg.get("model_type")
@@ -56,7 +59,7 @@ def resolve_architecture(cfg: dict) -> Architecture:
             if mt in arch.model_types:
                 return arch
     raise ConfigError(
-        f"unknown architecture: architectures={cfg.get('architectures')!r}, "
+        f"unknown architecture: architectures={named!r}, "
         f"model_type={cfg.get('model_type')!r}; registered: {sorted(ARCHITECTURES)}")
 
 

@@ -28,6 +28,29 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """Layer norm over the last axis: (x - mean) / sqrt(var + eps) * gain + bias, var the mean of
+    the squared deviations.  ``streams`` > 1: the input holds that many residual streams per
+    token and the norm reads their plain sum."""
+    size: int
+    eps: float
+    weight: str
+    bias: Optional[str]
+    streams: int = 1
+    kind: str = "layernorm"
+
+
+@dataclass(frozen=True)
+class ShortConvSpec:
+    """x_t + sum_j w[:, j] x_(t - taps + 1 + j): a causal convolution over time on each channel,
+    zeros before a sequence's start; the last ``taps - 1`` rows are a request's state."""
+    size: int
+    taps: int
+    weight: str                      # [size, taps]
+    kind: str = "short_conv"
+
+
+@dataclass(frozen=True)
 class RotarySpec:
     """Rotate-half rotary encoding of the first ``rotary_dim`` channels of a head."""
     head_dim: int
@@ -54,6 +77,30 @@ class AttentionSpec:
     position: Any                    # a position-encoding spec
     names: Dict[str, str]            # roles q, k, v, o -> checkpoint names
     kind: str = "attention"
+    # what follows is optional; a model that uses none of it runs as before
+    value_dim: Optional[int] = None          # size of a head's values (None: head_dim)
+    q_norm: Optional[str] = None             # gain [head_dim] of an RMS norm over each query head, before rotation
+    k_norm: Optional[str] = None             # the same for key heads
+    norm_eps: float = 1e-6
+    head_scale: Optional[str] = None         # [num_heads]: a number per query head that multiplies its scores
+    value_rotation: Optional[float] = None   # base: values are cached turned by their position over all their
+    #                                          channels (pair m by pos * base^(-2m/value_dim)), outputs turned back
+    value_pairs_interleaved: bool = False    # pairs (2m, 2m + 1) instead of (m, m + value_dim / 2)
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A recurrent mixer with a matrix state per head (mLSTM): exponential input gate, sigmoid
+    forget gate in the log domain, both capped as cap * tanh(x / cap), a running maximum that
+    starts at 0; per-head unit RMS of the read-out, a gain, a sigmoid output gate."""
+    hidden_size: int
+    num_heads: int
+    key_dim: int                     # per head, queries and keys
+    value_dim: int                   # per head
+    gate_cap: float
+    eps: float                       # of the read-out's unit RMS
+    names: Dict[str, str]            # roles q, k, v, gate, o, norm, i, i_bias, f, f_bias
+    kind: str = "mlstm"
 
 
 @dataclass(frozen=True)
@@ -84,12 +131,29 @@ class BlockSpec:
 
 
 @dataclass(frozen=True)
+class StreamsBlockSpec:
+    """One layer over ``streams`` residual streams (hyper-connections).  Sublayer q (1: the
+    mixer, 2: the feed-forward, which may be absent) reads u = sum_s in_q[s] x_s, computes
+    y = sublayer(norm_q(u)) and writes x_r <- sum_s mix_q[s, r] x_s + out_q[r] y, every stream from
+    the old ones.  ``conv``: a short convolution over time between the first norm and the mixer.
+    ``streams`` None: one stream and the plain residual sum x <- x + y (no weights)."""
+    streams: Optional[int]
+    mixer: Any
+    ffn: Any                         # None: the layer has no second sublayer
+    norms: Dict[str, Any]            # pre_mixer, pre_ffn
+    conv: Any                        # ShortConvSpec or None
+    names: Dict[str, str]            # in1, out1, mix1, in2, out2, mix2 (absent without streams)
+    kind: str = "streams"
+
+
+@dataclass(frozen=True)
 class EmbeddingSpec:
     vocab_size: int
     hidden_size: int
     scale: float                     # multiplies the gathered row
     weight: str
     kind: str = "embedding"
+    copies: int = 1                  # the row is written this many times (one per residual stream)
 
 
 @dataclass(frozen=True)
@@ -134,7 +198,7 @@ class ModelPlan:
         for i, call in enumerate(self.order):
             b = self.layers[call.layer]
             win = getattr(b.mixer, "window", None)
-            out.append(f"call {i}: layer {call.layer} {b.arrangement} mixer={b.mixer.kind}"
-                       f"(window={win}) ffn={b.ffn.kind}"
+            out.append(f"call {i}: layer {call.layer} {getattr(b, 'arrangement', b.kind)} mixer={b.mixer.kind}"
+                       f"(window={win}) ffn={getattr(b.ffn, 'kind', None)}"
                        + (f" cache_of={call.cache_of}" if call.cache_of is not None else ""))
         return out

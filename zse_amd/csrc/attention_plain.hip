@@ -20,16 +20,16 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
     const act_t* __restrict__ q, int q_stride, const act_t* __restrict__ kcache,
     const act_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ req_of_token, const int* __restrict__ positions,
-    act_t* __restrict__ out, int nh, int nkv, int hd, int bs, float scale, float softcap,
-    int window, int v_transposed) {
+    act_t* __restrict__ out, int nh, int nkv, int hd, int vd, int bs, float scale, float softcap,
+    int window, int v_transposed, const float* __restrict__ v_freq, int v_interleaved) {
   __shared__ float sq[AP_MAX_HD];
   __shared__ float sp[64];
   __shared__ int spage[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
-  act_t* o = out + ((size_t)t * nh + h) * hd;
+  act_t* o = out + ((size_t)t * nh + h) * vd;
   if (pos < 0) {  // padding row
-    for (int d = lane; d < hd; d += 64) o[d] = from_f32<act_t>(0.f);
+    for (int d = lane; d < vd; d += 64) o[d] = from_f32<act_t>(0.f);
     return;
   }
   const int r = req_of_token[t];
@@ -67,15 +67,15 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
 #pragma unroll
     for (int c = 0; c < AP_MAX_HD / 64; c++) {
       const int d = lane + c * 64;
-      if (d < hd) {
+      if (d < vd) {
         float a = acc[c] * corr;
         for (int jj = 0; jj < 64; jj++) {
           const int pg = spage[jj];
           if (pg < 0) continue;
-          const size_t head_base = ((size_t)pg * nkv + kvh) * bs * hd;
+          const size_t head_base = ((size_t)pg * nkv + kvh) * bs * vd;
           const size_t off = (j0 + jj) % bs;
           const act_t v = v_transposed ? vcache[head_base + (size_t)d * bs + off]
-                                       : vcache[head_base + off * hd + d];
+                                       : vcache[head_base + off * vd + d];
           a = fmaf(sp[jj], to_f32(v), a);
         }
         acc[c] = a;
@@ -83,22 +83,46 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
     }
   }
   const float inv = 1.f / l;
+  if (v_freq == nullptr) {
+#pragma unroll
+    for (int c = 0; c < AP_MAX_HD / 64; c++) {
+      const int d = lane + c * 64;
+      if (d < vd) o[d] = from_f32<act_t>(acc[c] * inv);
+    }
+    return;
+  }
+  // values were turned by their own positions when they were stored: the sum is turned back
+  // by the query's position, pair m by -pos * v_freq[m]
+  __syncthreads();
 #pragma unroll
   for (int c = 0; c < AP_MAX_HD / 64; c++) {
     const int d = lane + c * 64;
-    if (d < hd) o[d] = from_f32<act_t>(acc[c] * inv);
+    if (d < vd) sq[d] = acc[c] * inv;
+  }
+  __syncthreads();
+  const int half = vd / 2;
+  for (int m2 = lane; m2 < half; m2 += 64) {
+    float sn, cs, ra, rb;
+    sincosf(-(float)pos * v_freq[m2], &sn, &cs);
+    const int ia = v_interleaved ? 2 * m2 : m2, ib = v_interleaved ? 2 * m2 + 1 : m2 + half;
+    rotate_pair(sq[ia], sq[ib], sn, cs, ra, rb);
+    o[ia] = from_f32<act_t>(ra);
+    o[ib] = from_f32<act_t>(rb);
   }
 }
 
 // softcap <= 0: no cap; window <= 0: every earlier key is visible.  v_transposed: V is
 // cached as [page][kv head][hd][bs] instead of [page][kv head][bs][hd].
-extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcache, const void* vcache,
-                                  const int* block_table, int max_blocks, const int* req_of_token,
-                                  const int* positions, void* out, int T, int nh, int nkv, int hd,
-                                  int bs, float scale, float softcap, int window, int v_transposed,
-                                  void* stream) {
-  ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0 && max_blocks > 0,
+// hd: the size of a head's queries and keys; vd: of its values (the output's too).  v_freq (may
+// be null): float [vd / 2], values are cached turned by their positions and the output is turned back.
+extern "C" int zk_attention_plain_ext(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                      const int* block_table, int max_blocks, const int* req_of_token,
+                                      const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
+                                      int bs, float scale, float softcap, int window, int v_transposed,
+                                      const float* v_freq, int v_interleaved, void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && bs > 0 && max_blocks > 0,
              "zk_attention_plain: bad sizes");
+  ZK_REQUIRE(vd <= AP_MAX_HD && (v_freq == nullptr || vd % 2 == 0), "zk_attention_plain: value size above 256, or odd with a rotation");
   ZK_REQUIRE(nh % nkv == 0, "zk_attention_plain: heads must be a multiple of kv heads");
   ZK_REQUIRE(hd <= AP_MAX_HD, "zk_attention_plain: head_dim above 256 is not supported");
   ZK_REQUIRE(nh <= 65535, "zk_attention_plain: too many heads");
@@ -107,6 +131,22 @@ extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcach
   dim3 grid(T, nh);
   attention_plain_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(
       (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
-      req_of_token, positions, (act_t*)out, nh, nkv, hd, bs, scale, softcap, window, v_transposed);
+      req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
+      v_interleaved);
   return zk_launch_status("zk_attention_plain");
 }
+
+extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                  const int* block_table, int max_blocks, const int* req_of_token,
+                                  const int* positions, void* out, int T, int nh, int nkv, int hd,
+                                  int bs, float scale, float softcap, int window, int v_transposed,
+                                  void* stream) {
+  return zk_attention_plain_ext(q, q_stride, kcache, vcache, block_table, max_blocks, req_of_token, positions, out, T,
+                                nh, nkv, hd, hd, bs, scale, softcap, window, v_transposed, nullptr, 0, stream);
+}
+
+#include "packed_call.h"
+extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
+static const int attention_plain_ext_entered = zk_steplist_register(
+    "zk_attention_plain_ext", zk_packed::Call<zk_attention_plain_ext>::nargs,
+    (void*)zk_packed::Call<zk_attention_plain_ext>::call);

@@ -437,7 +437,7 @@ __global__ void gated_act_kernel(const act_t* __restrict__ gu, act_t* __restrict
   if (i >= I) return;
   const float g = to_f32(gu[(size_t)t * 2 * I + i]);
   const float u = to_f32(gu[(size_t)t * 2 * I + I + i]);
-  const float a = act == 0 ? gelu_tanh(g) : silu(g);
+  const float a = act == 0 ? gelu_tanh(g) : act == 1 ? silu(g) : fmaxf(g, 0.f);
   out[(size_t)t * I + i] = from_f32<act_t>(a * u);
 }
 
@@ -822,7 +822,7 @@ int zk_norm_add_norm(const void* sub, int sub_parts, const float* w_post, float 
 
 // act: 0 = gelu_tanh, 1 = silu
 int zk_gated_act(const void* gu, void* out, int T, int I, int act, void* stream) {
-  ZK_REQUIRE(T >= 0 && I > 0 && (act == 0 || act == 1), "zk_gated_act: bad arguments");
+  ZK_REQUIRE(T >= 0 && I > 0 && act >= 0 && act <= 2, "zk_gated_act: bad arguments");
   ZK_REQUIRE(T <= 65535, "zk_gated_act: more than 65535 rows");
   if (T == 0) return 0;
   dim3 grid((I + 255) / 256, T);

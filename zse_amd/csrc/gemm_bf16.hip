@@ -53,7 +53,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // <= 0: none) and that value's column in ``partials`` [M][strips] as (float, int), larger value
 // first, equal values to the lower column, NaN never, which a joining kernel reduces to one
 // column a row: the greedy choice without the logits ever reaching memory.
-enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4 };
+enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4, EPI_RELU = 5 };
 
 struct Pick {
   float value;
@@ -96,6 +96,7 @@ __device__ __forceinline__ float epi_gelu_tanh(float g) {
   return g * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
 }
 __device__ __forceinline__ float epi_gate(float g, float u, int epi) {
+  if (epi == EPI_RELU) return fmaxf(g, 0.f) * u;
   return (epi == EPI_GELU_TANH ? epi_gelu_tanh(g) : g / (1.0f + expf(-g))) * u;
 }
 
@@ -1353,7 +1354,7 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
   return zk_launch_status("zk_strip_layout");
 }
 
-// epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate.  For the gated
+// epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate, 5 relu gate.  For the gated
 // epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
 // w_strip: W is in strip layout (zk_strip_layout), which needs K % 32 == 0 and, for the
 // gated epilogues, N % 16 == 0.
@@ -1422,10 +1423,10 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
-  ZK_REQUIRE(epi >= 0 && epi <= EPI_PICK, "zk_gemm_bf16: unknown epilogue");
+  ZK_REQUIRE(epi >= 0 && epi <= EPI_RELU, "zk_gemm_bf16: unknown epilogue");
   ZK_REQUIRE(epi != EPI_SOFTCAP || cap > 0.f, "zk_gemm_bf16: soft cap must be positive");
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
-  const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU;
+  const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU || epi == EPI_RELU;
   ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
   if (parts) *parts = 0;
   if (M == 0) return 0;

@@ -1,0 +1,106 @@
+// What happens to a step's queries, keys and values between their product and the attention:
+// an optional norm over each query and key head, an optional number per query head, the rotary
+// encoding of queries and keys, an optional rotation of the values, and the store of keys and
+// values into the paged cache.  One wave per (token, head).
+//
+//   q_h <- rot_p( q_h / sqrt(mean(q_h^2) + eps) * gq ) * c_h          (k likewise with gk, no c)
+//   v_g <- rot'_p( v_g )
+//
+// rot_p turns pair (i, i + dims/2) of the first ``dims`` channels by p * inv_freq[i]; rot'_p turns
+// pair m of all value channels ((m, m + E/2), or (2m, 2m + 1) when interleaved) by p * v_freq[m].
+// A row of the input holds nh query heads of D, then nkv key heads of D, then nkv value heads of
+// E (the last two absent when the mixer reads another one's cache).  All arithmetic is float; a
+// value is rounded to the activation type once, when it is stored.
+#include "common.h"
+#include "packed_call.h"
+
+extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
+
+#define HP_MAX 256
+
+__global__ __launch_bounds__(64) void head_prep_kernel(
+    act_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slot_map,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, const float* __restrict__ head_scale, float eps,
+    const float* __restrict__ inv_freq, int rot_dims, const float* __restrict__ v_freq, int v_interleaved,
+    act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh, int nkv, int D, int E, int bs, int v_transposed) {
+  __shared__ float buf[HP_MAX];
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int pos = positions[t];
+  if (pos < 0) return;                                   // a padding row
+  const size_t width = (size_t)(nh + nkv) * D + (size_t)nkv * E;
+  const int kind = head < nh ? 0 : head < nh + nkv ? 1 : 2;
+  const int size = kind == 2 ? E : D;
+  const size_t at = (size_t)t * width + (kind == 2 ? (size_t)(nh + nkv) * D + (size_t)(head - nh - nkv) * E : (size_t)head * D);
+  const int slot = (kind != 0 && slot_map) ? slot_map[t] : -1;
+  if (kind != 0 && slot < 0) return;
+  float sum = 0.f;
+  for (int d = lane; d < size; d += 64) {
+    const float x = to_f32(qkv[at + d]);
+    buf[d] = x;
+    sum = fmaf(x, x, sum);
+  }
+  const float* gain = kind == 0 ? q_gain : kind == 1 ? k_gain : nullptr;
+  if (gain != nullptr) {
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sqrtf(sum / (float)size + eps);
+    const float c = (kind == 0 && head_scale) ? head_scale[head] : 1.f;
+    for (int d = lane; d < size; d += 64) buf[d] = buf[d] * inv * gain[d] * c;
+  } else if (kind == 0 && head_scale) {
+    const float c = head_scale[head];
+    for (int d = lane; d < size; d += 64) buf[d] *= c;
+  }
+  __syncthreads();
+  // rotation: every lane takes whole pairs, so nothing is read after another lane wrote it
+  const float* freq = kind == 2 ? v_freq : inv_freq;
+  const int dims = kind == 2 ? (v_freq ? E : 0) : (inv_freq ? rot_dims : 0);
+  const bool inter = kind == 2 && v_interleaved;
+  const int half = dims / 2;
+  for (int m = lane; m < half; m += 64) {
+    float sn, cs, ra, rb;
+    sincosf((float)pos * freq[m], &sn, &cs);
+    const int ia = inter ? 2 * m : m, ib = inter ? 2 * m + 1 : m + half;
+    rotate_pair(buf[ia], buf[ib], sn, cs, ra, rb);
+    buf[ia] = ra;
+    buf[ib] = rb;
+  }
+  __syncthreads();
+  if (kind == 0) {
+    for (int d = lane; d < size; d += 64) qkv[at + d] = from_f32<act_t>(buf[d]);
+    return;
+  }
+  const size_t page = slot / bs, off = slot % bs;
+  if (kind == 1) {
+    act_t* dst = kcache + ((page * nkv + (head - nh)) * bs + off) * D;
+    for (int d = lane; d < size; d += 64) dst[d] = from_f32<act_t>(buf[d]);
+  } else if (v_transposed) {
+    act_t* dst = vcache + (page * nkv + (head - nh - nkv)) * (size_t)E * bs + off;
+    for (int d = lane; d < size; d += 64) dst[(size_t)d * bs] = from_f32<act_t>(buf[d]);
+  } else {
+    act_t* dst = vcache + ((page * nkv + (head - nh - nkv)) * bs + off) * E;
+    for (int d = lane; d < size; d += 64) dst[d] = from_f32<act_t>(buf[d]);
+  }
+}
+
+// nkv: key/value heads held in the rows (0 for a mixer that stores none).  q_gain, k_gain,
+// head_scale, inv_freq, v_freq may each be null (the step it stands for is then left out).
+extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
+                            const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
+                            int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
+                            int nh, int nkv, int D, int E, int bs, int v_transposed, void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && D > 0 && E > 0 && bs > 0, "zk_head_prep: bad sizes");
+  ZK_REQUIRE(D <= HP_MAX && E <= HP_MAX, "zk_head_prep: heads of more than 256 channels are not supported");
+  ZK_REQUIRE(inv_freq == nullptr || (rot_dims % 2 == 0 && rot_dims >= 0 && rot_dims <= D),
+             "zk_head_prep: the rotated channels must be even in number and at most the head's");
+  ZK_REQUIRE(v_freq == nullptr || E % 2 == 0, "zk_head_prep: rotated values need an even size");
+  ZK_REQUIRE(nkv == 0 || (kcache != nullptr && vcache != nullptr && slot_map != nullptr), "zk_head_prep: no cache to store into");
+  ZK_REQUIRE(nh + 2 * nkv <= 65535, "zk_head_prep: too many heads");
+  if (T == 0) return 0;
+  dim3 grid(T, nh + 2 * nkv);
+  head_prep_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, q_gain, k_gain, head_scale, eps,
+                                                         inv_freq, rot_dims, v_freq, v_interleaved, (act_t*)kcache,
+                                                         (act_t*)vcache, nh, nkv, D, E, bs, v_transposed);
+  return zk_launch_status("zk_head_prep");
+}
+
+static const int head_prep_entered =
+    zk_steplist_register("zk_head_prep", zk_packed::Call<zk_head_prep>::nargs, (void*)zk_packed::Call<zk_head_prep>::call);

@@ -1,7 +1,7 @@
 """A model: the parts a plan names, built, loaded and run in the plan's order."""
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field, replace
 from typing import Dict, List, Optional
 
 from .. import parts as _parts  # noqa: F401  (registers the built-in part kinds)
@@ -20,6 +20,8 @@ class CallCache:
     v_transposed: bool = False
     state_offset: int = 0            # byte offset inside a request's state slot
     state_bytes: int = 0
+    shared: bool = False             # k, v and group are another entry's (this entry stores none)
+    extra: Dict[str, tuple] = field(default_factory=dict)   # states of the layer's other parts: key -> (offset, bytes)
 
 
 class Model:
@@ -64,6 +66,15 @@ class Model:
                 out.append(None)
             else:
                 out.append(self.blocks[call.layer].mixer.cache_need())
+        # keys that another entry reads too must stay as long as the widest window among the
+        # readers needs them (for ever, if one of them sees every key)
+        for i, call in enumerate(self.plan.order):
+            own = out[call.cache_of] if call.cache_of is not None else None
+            if isinstance(own, PagedKV):
+                reader = self.blocks[call.layer].mixer.cache_need()
+                if isinstance(reader, PagedKV) and own.window is not None and \
+                        (reader.window is None or reader.window > own.window):
+                    out[call.cache_of] = replace(own, window=reader.window)
         return out
 
     # ---- what a step costs, for measurements: read off the parts, whatever the architecture
@@ -94,7 +105,7 @@ class Model:
         for need in self.cache_needs():
             if isinstance(need, PagedKV):
                 seen = min(context, need.window) if need.window else context
-                total += 2 * need.num_kv_heads * need.head_dim * seen * itemsize
+                total += need.num_kv_heads * (need.head_dim + (need.value_dim or need.head_dim)) * seen * itemsize
         return total
 
     def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor, pick=None):
@@ -111,7 +122,7 @@ class Model:
         x = None
         base = ctx.arena.mark()
         for i, call in enumerate(order):
-            cache = caches[call.cache_of if call.cache_of is not None else i]
+            cache = caches[i] if caches[i].shared else caches[call.cache_of if call.cache_of is not None else i]
             blk = self.blocks[call.layer]
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
             if hasattr(blk, "entry_norm"):

@@ -48,7 +48,7 @@ def main(argv: Optional[list] = None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
-    ap.add_argument("--max-seqs", type=int, default=8)
+    ap.add_argument("--max-seqs", type=int, default=4, help="state slots: the most requests live at a time")
     ap.add_argument("--plain", action="store_true",
                     help="bfloat16 only: the plain kernels instead of the tuned ones")
     a = ap.parse_args(argv)

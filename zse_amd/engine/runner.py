@@ -180,6 +180,7 @@ class StepRunner:
         item = ITEMSIZE[self.dtype]
         for i, need in enumerate(needs):
             cc = CallCache(need=need)
+            call = model.plan.order[i]
             if isinstance(need, PagedKV):
                 cc.group = gid_of[i]
                 # page 0 of every slab is the runner's own: cleared here, never handed out and
@@ -187,16 +188,29 @@ class StepRunner:
                 pages = groups[cc.group].num_pages + 1
                 shape = (pages, need.num_kv_heads, self.page_size, need.head_dim)
                 cc.k = rt.zeros(shape, self.dtype)
-                mixer = model.blocks[model.plan.order[i].layer].mixer
+                mixer = model.blocks[call.layer].mixer
                 cc.v_transposed = bool(self.tuned and getattr(mixer, "wants_v_transposed", None) and
                                        mixer.wants_v_transposed(self.k, self.dtype, self.page_size))
+                vd = need.value_dim or need.head_dim
+                shape = (pages, need.num_kv_heads, self.page_size, vd)
                 if cc.v_transposed:
-                    shape = (pages, need.num_kv_heads, need.head_dim, self.page_size)
+                    shape = (pages, need.num_kv_heads, vd, self.page_size)
                 cc.v = rt.zeros(shape, self.dtype)
             elif isinstance(need, StateNeed):
                 cc.state_offset = slot_bytes
                 cc.state_bytes = int(need.nbytes)
                 slot_bytes += (int(need.nbytes) + 15) // 16 * 16
+            elif call.cache_of is not None:
+                # the entry reads another entry's keys and values: the same slabs and tables,
+                # beside whatever state of its own it keeps
+                own = self.caches[call.cache_of]
+                cc.need, cc.group, cc.k, cc.v, cc.v_transposed = own.need, own.group, own.k, own.v, own.v_transposed
+                cc.shared = True
+            # what the layer's other parts keep per request (a convolution's last rows, say)
+            block = model.blocks[call.layer]
+            for key, nbytes in (block.state_needs() if hasattr(block, "state_needs") else []):
+                cc.extra[key] = (slot_bytes, int(nbytes))
+                slot_bytes += (int(nbytes) + 15) // 16 * 16
             self.caches.append(cc)
         self.slot_bytes = slot_bytes
         self.manager = CacheManager(groups, self.page_size, self.max_seqs, self.max_model_len, slot_bytes,
@@ -205,7 +219,7 @@ class StepRunner:
         # clears a page in all of them
         self._slabs = []
         for gid in range(len(groups)):
-            ts = [t for cc in self.caches if cc.group == gid and cc.k is not None for t in (cc.k, cc.v)]
+            ts = [t for cc in self.caches if cc.group == gid and cc.k is not None and not cc.shared for t in (cc.k, cc.v)]
             ptrs = rt.upload(np.array([t.ptr for t in ts], dtype=np.uint64).view(np.float64), "float64")
             sizes = rt.upload(np.array([t.nbytes // t.shape[0] for t in ts], dtype=np.uint64).view(np.float64), "float64")
             self._slabs.append((ptrs, sizes, len(ts)))
@@ -271,7 +285,7 @@ class StepRunner:
         return 4 * T + (R + 1) + 4 * R + G * (T + R * self.max_blocks) + 64
 
     def cache_bytes(self) -> int:
-        return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None)
+        return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None and not c.shared)
 
     # ------------------------------------------------------------------ requests
     def _clear_slot(self, req, slot: int) -> None:

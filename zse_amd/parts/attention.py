@@ -15,8 +15,10 @@ from __future__ import annotations
 
 from typing import List
 
+import numpy as np
+
 from ..runtime.device import BF16, Tensor
-from .base import PagedKV, Part, TensorReq, build_part, register_part
+from .base import ROLE_GAIN, PagedKV, Part, TensorReq, build_part, register_part
 from .ops import linear, tuned_gemm
 
 
@@ -27,11 +29,24 @@ class PagedAttention(Part):
         s = self.spec = spec
         if s.num_heads % s.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
-        if s.head_dim % 16 or s.head_dim > 256:
-            raise ValueError(f"head_dim must be a multiple of 16 up to 256, got {s.head_dim}")
+        if s.head_dim > 256 or s.head_dim < 1:
+            raise ValueError(f"head_dim must lie in 1..256, got {s.head_dim}")
         self.position = build_part("position", s.position)
         self.shared_kv = "k" not in s.names        # reads another call's cache, writes none
         self.w_qkv = self.w_o = None
+        # optional steps between the product and the attention (see AttentionSpec): any of them
+        # sends the mixer down the general path, whose kernels take them all as parameters
+        self.value_dim = int(getattr(s, "value_dim", None) or s.head_dim)
+        self.q_norm_name, self.k_norm_name = getattr(s, "q_norm", None), getattr(s, "k_norm", None)
+        self.head_scale_name = getattr(s, "head_scale", None)
+        self.value_base = getattr(s, "value_rotation", None)
+        self.general = bool(self.value_dim != s.head_dim or self.q_norm_name or self.k_norm_name or
+                            self.head_scale_name or self.value_base)
+        if self.value_dim > 256:
+            raise ValueError(f"value_dim up to 256, got {self.value_dim}")
+        if self.value_base and self.value_dim % 2:
+            raise ValueError(f"rotated values need an even value_dim, got {self.value_dim}")
+        self.q_gain = self.k_gain = self.head_scale = self.value_freq = None
         self.decode_chunk = 64                     # keys a wave of the split decode attention takes
 
     def children(self):
@@ -39,35 +54,52 @@ class PagedAttention(Part):
 
     def tensor_reqs(self) -> List[TensorReq]:
         s = self.spec
-        q = TensorReq(s.names["q"], (s.num_heads * s.head_dim, s.hidden_size))
-        o = TensorReq(s.names["o"], (s.hidden_size, s.num_heads * s.head_dim))
+        out = [TensorReq(s.names["q"], (s.num_heads * s.head_dim, s.hidden_size)),
+               TensorReq(s.names["o"], (s.hidden_size, s.num_heads * self.value_dim))]
+        if self.q_norm_name:
+            out.append(TensorReq(self.q_norm_name, (s.head_dim,), ROLE_GAIN))
+        if self.head_scale_name:
+            out.append(TensorReq(self.head_scale_name, (s.num_heads,), ROLE_GAIN))
         if self.shared_kv:
-            return [q, o]
-        kv = (s.num_kv_heads * s.head_dim, s.hidden_size)
-        return [q, TensorReq(s.names["k"], kv), TensorReq(s.names["v"], kv), o]
+            return out
+        out += [TensorReq(s.names["k"], (s.num_kv_heads * s.head_dim, s.hidden_size)),
+                TensorReq(s.names["v"], (s.num_kv_heads * self.value_dim, s.hidden_size))]
+        if self.k_norm_name:
+            out.append(TensorReq(self.k_norm_name, (s.head_dim,), ROLE_GAIN))
+        return out
 
     def load(self, weights, rt, dtype):
         s = self.spec
         names = [s.names["q"]] if self.shared_kv else [s.names[r] for r in ("q", "k", "v")]
         strip = getattr(weights, "wants_strip", None)
         self.w_qkv = weights.matrix(names, strip=True) if strip and strip(s.hidden_size) else weights.matrix(names)
-        o_cols = s.num_heads * s.head_dim
+        o_cols = s.num_heads * self.value_dim
         self.w_o = (weights.matrix([s.names["o"]], strip=True) if strip and strip(o_cols)
                     else weights.matrix([s.names["o"]]))
+        if self.q_norm_name:
+            self.q_gain = weights.vector(self.q_norm_name)
+        if self.k_norm_name and not self.shared_kv:
+            self.k_gain = weights.vector(self.k_norm_name)
+        if self.head_scale_name:
+            self.head_scale = weights.vector(self.head_scale_name)
+        if self.value_base:
+            m = np.arange(self.value_dim // 2, dtype=np.float64)
+            self.value_freq = rt.upload(np.power(float(self.value_base), -2.0 * m / self.value_dim).astype(np.float32))
 
     def cache_need(self):
         s = self.spec
-        return PagedKV(s.num_kv_heads, s.head_dim, s.window)
+        return PagedKV(s.num_kv_heads, s.head_dim, s.window,
+                       self.value_dim if self.value_dim != s.head_dim else None)
 
     def flops_per_key(self) -> float:
-        return 4.0 * self.spec.num_heads * self.spec.head_dim        # q.k and p.v
+        return 2.0 * self.spec.num_heads * (self.spec.head_dim + self.value_dim)        # q.k and p.v
 
     PORTION_RANGES_BYTES = 192 << 20
 
     def wants_v_transposed(self, kernels, dtype: str, page_size: int) -> bool:
         """The matrix-core kernel reads V as [page][kv head][hd][bs]."""
         s = self.spec
-        return bool(dtype == BF16 and kernels.has("zk_attention_bf16") and
+        return bool(dtype == BF16 and self.value_dim == s.head_dim and kernels.has("zk_attention_bf16") and
                     kernels.zk_attention_bf16_supports(s.num_heads, s.num_kv_heads, s.head_dim, page_size))
 
     def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size, max_batch_tokens=0) -> int:
@@ -104,7 +136,46 @@ class PagedAttention(Part):
         ``head_dim`` wide.  Everything else of the mixer stays as it is; the product that
         rotates and stores its own results is then not used, since this step lies in between."""
 
+    def _forward_general(self, ctx, x: Tensor, cache) -> Tensor:
+        """The path of a mixer with head norms, a number per head, values of their own size or
+        rotated values: product, one kernel for everything up to the cache, attention, and
+        the turning back of the output where values are stored rotated."""
+        s, k = self.spec, ctx.k
+        T = x.shape[0]
+        nh, nkv, hd, vd = s.num_heads, s.num_kv_heads, s.head_dim, self.value_dim
+        n_store = 0 if self.shared_kv else nkv
+        width = (nh + n_store) * hd + n_store * vd
+        g = ctx.group(cache.group)
+        tables = self.position.rotary_tables()
+        qkv = linear(ctx, x, self.w_qkv, ctx.alloc((T, width)))
+        if tables is None:
+            self.position.apply(ctx, qkv, nh, n_store, hd)
+        ptr = lambda t: t.ptr if t is not None else None
+        vfreq = ptr(self.value_freq)
+        inter = 1 if getattr(s, "value_pairs_interleaved", False) else 0
+        k.zk_head_prep(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain), ptr(self.k_gain),
+                       ptr(self.head_scale), float(s.norm_eps), tables[0].ptr if tables is not None else None,
+                       tables[1] if tables is not None else 0, vfreq, inter, cache.k.ptr, cache.v.ptr, T, nh, n_store,
+                       hd, vd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+        o = ctx.alloc((T, nh * vd))
+        cap = float(s.softcap) if s.softcap else 0.0
+        win = int(s.window) if s.window else 0
+        if cache.v_transposed and ctx.tuned and vd == hd:
+            k.zk_attention_bf16(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
+                                ctx.q_start, ctx.ctx_len, o.ptr, ctx.R, ctx.n_multi, ctx.max_q_len,
+                                ctx.max_ctx, nh, nkv, hd, g.page_size, s.scale, cap, win,
+                                self.decode_chunk, ctx.workspace.ptr, ctx.workspace.nbytes, ctx.stream)
+            if vfreq is not None:
+                k.zk_rotate_heads(o.ptr, ctx.positions, vfreq, T, nh, vd, inter, -1.0, ctx.stream)
+        else:
+            k.zk_attention_plain_ext(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
+                                     ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv, hd, vd, g.page_size, s.scale,
+                                     cap, win, 1 if cache.v_transposed else 0, vfreq, inter, ctx.stream)
+        return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
+
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
+        if self.general:
+            return self._forward_general(ctx, x, cache)
         s, k = self.spec, ctx.k
         T = x.shape[0]
         nh, nkv, hd = s.num_heads, s.num_kv_heads, s.head_dim

@@ -18,6 +18,10 @@ Interfaces, by slot:
             forward(ctx, x, cache) -> Tensor[T, hidden]
   ffn       forward(ctx, x) -> Tensor[T, hidden]
   block     forward(ctx, h, cache): updates the float stream ``h`` in place.
+            state_needs() -> [(key, bytes)] (optional): what its parts other than the mixer
+            keep per request; their places in the state slot come as ``cache.extra[key]``.
+  filter    forward(ctx, x, state_offset) -> Tensor like x: something over time between a norm
+            and a mixer (a short convolution); state_bytes() says what it keeps per request.
 """
 from __future__ import annotations
 
@@ -43,6 +47,7 @@ class PagedKV:
     num_kv_heads: int
     head_dim: int
     window: Optional[int]
+    value_dim: Optional[int] = None     # size of a head's values where it differs from its keys'
 
 
 @dataclass(frozen=True)
@@ -92,7 +97,7 @@ class Part:
 
 
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {
-    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {},
+    "norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}, "embedding": {}, "head": {}, "filter": {},
 }
 
 

@@ -47,9 +47,13 @@ class Embedding(Part):
 
     def forward(self, ctx) -> Tensor:
         s = self.spec
-        h = ctx.alloc((ctx.T, s.hidden_size), F32)
-        ctx.k.zk_embed(self.table.ptr, ctx.tokens, h.ptr, self.scale, ctx.T, s.hidden_size,
+        copies = int(getattr(s, "copies", 1))
+        h = ctx.alloc((ctx.T, copies * s.hidden_size), F32)
+        row = h if copies == 1 else ctx.alloc((ctx.T, s.hidden_size), F32)
+        ctx.k.zk_embed(self.table.ptr, ctx.tokens, row.ptr, self.scale, ctx.T, s.hidden_size,
                        s.vocab_size, 1 if self.table.layout == "strip" else 0, ctx.stream)
+        if copies > 1:          # every residual stream starts as the embedded row
+            ctx.k.zk_replicate(row.ptr, h.ptr, ctx.T, copies, s.hidden_size, ctx.stream)
         return h
 
 

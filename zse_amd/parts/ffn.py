@@ -1,5 +1,6 @@
 """Gated feed-forward: act(x Wg^T) * (x Wu^T), then Wd^T.
 
+act is one of gelu_tanh, silu and relu (max(z, 0)).
 gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) is the
 reference's GeGLU kernel (orchestrator/kernels.py:1678-1697, wiring
 model_runner.py:518-530); silu is its Llama activation (kernels.py:228-244).
@@ -13,7 +14,7 @@ from ..runtime.device import Tensor
 from .base import Part, TensorReq, register_part
 from .ops import linear, tuned_gemm
 
-ACTIVATION_CODES = {"gelu_tanh": 0, "silu": 1}
+ACTIVATION_CODES = {"gelu_tanh": 0, "silu": 1, "relu": 2}
 
 
 class GatedMLP(Part):

@@ -1,0 +1,76 @@
+"""A recurrent mixer with a matrix memory per head (the mLSTM of xLSTM).
+
+Per head, D query/key channels and E value channels; the state (S [D, E], n [D], m) starts
+at zero and is carried as floats in the request's state slot:
+
+    i_t = cap tanh((W_i x_t + b_i) / cap)          f_t = logsigmoid(cap tanh((W_f x_t + b_f) / cap))
+    m_t = max(f_t + m_(t-1), i_t)
+    S_t = exp(f_t + m_(t-1) - m_t) S_(t-1) + exp(i_t - m_t) k_t v_t^T      (n_t likewise with k_t)
+    o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6),    q_t = W_q x_t D^(-1/2)
+    out = W_o ( o_t / sqrt(mean(o_t^2) + eps) * g * sigmoid(W_z x_t) )      (the mean per head)
+
+q, k, v and z are one product; the two gates are a second, small one whose results stay float.
+"""
+from __future__ import annotations
+
+from typing import List
+
+from ..runtime.device import F32, Tensor
+from .base import ROLE_GAIN, Part, StateNeed, TensorReq, register_part
+from .ops import linear
+
+
+class MatrixMemory(Part):
+    graph_safe = True      # rows, requests and slots are read by the kernel from device memory
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.value_dim > 256:
+            raise ValueError(f"up to 256 value channels a head, got {s.value_dim}")
+        if not s.gate_cap > 0:
+            raise ValueError(f"the gates' cap must be positive, got {s.gate_cap}")
+        self.w_qkvz = self.w_gates = self.w_o = None
+        self.bias_i = self.bias_f = self.gain = None
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        s, n = self.spec, self.spec.names
+        H, D, E, W = s.num_heads, s.key_dim, s.value_dim, s.hidden_size
+        return [TensorReq(n["q"], (H * D, W)), TensorReq(n["k"], (H * D, W)), TensorReq(n["v"], (H * E, W)),
+                TensorReq(n["gate"], (H * E, W)), TensorReq(n["o"], (W, H * E)),
+                TensorReq(n["norm"], (H * E,), ROLE_GAIN),
+                TensorReq(n["i"], (H, W)), TensorReq(n["i_bias"], (H,), ROLE_GAIN),
+                TensorReq(n["f"], (H, W)), TensorReq(n["f_bias"], (H,), ROLE_GAIN)]
+
+    def load(self, weights, rt, dtype):
+        s, n = self.spec, self.spec.names
+        strip = getattr(weights, "wants_strip", None)
+        wide = bool(strip and strip(s.hidden_size))
+        self.w_qkvz = weights.matrix([n["q"], n["k"], n["v"], n["gate"]], strip=wide)
+        self.w_gates = weights.matrix([n["i"], n["f"]], strip=wide)
+        self.w_o = weights.matrix([n["o"]], strip=bool(strip and strip(s.num_heads * s.value_dim)))
+        self.bias_i, self.bias_f = weights.vector(n["i_bias"]), weights.vector(n["f_bias"])
+        self.gain = weights.vector(n["norm"])
+
+    def cache_need(self):
+        s = self.spec
+        return StateNeed(s.num_heads * (s.key_dim * s.value_dim + s.key_dim + 1) * 4)
+
+    def flops_per_token(self) -> float:
+        s = self.spec
+        return super().flops_per_token() + 4.0 * s.num_heads * s.key_dim * s.value_dim    # the state's update and read-out
+
+    def forward(self, ctx, x: Tensor, cache) -> Tensor:
+        s, k = self.spec, ctx.k
+        T = x.shape[0]
+        H, D, E = s.num_heads, s.key_dim, s.value_dim
+        ld = 2 * H * (D + E)
+        qkvz = linear(ctx, x, self.w_qkvz, ctx.alloc((T, ld)))
+        gates = linear(ctx, x, self.w_gates, ctx.alloc((T, 2 * H), F32))
+        out = ctx.alloc((T, H * E))
+        k.zk_mlstm(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, self.gain.ptr, ctx.state.ptr,
+                   ctx.state.shape[1], cache.state_offset // 4, ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, D, E,
+                   float(s.gate_cap), float(s.eps), ctx.stream)
+        return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
+
+
+register_part("mixer", "mlstm", MatrixMemory)

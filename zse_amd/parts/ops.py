@@ -6,7 +6,7 @@ import ctypes
 from ..runtime.device import BF16, F32, Tensor
 
 
-EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3}
+EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3, "relu": 5}
 
 
 def tuned_gemm(ctx, K: int) -> bool:
@@ -22,7 +22,7 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     ``out`` may be float32 (logits) or the activation type.  In the 32-bit
     library only the plain product exists; the bf16 library picks a matrix-core
     kernel by the number of rows.  ``epilogue`` (matrix-core product only):
-    "softcap" applies cap * tanh(x / cap); "gelu_tanh" / "silu" take w as
+    "softcap" applies cap * tanh(x / cap); "gelu_tanh" / "silu" / "relu" take w as
     [2N, K], gate rows first, and store act(gate) * up.
 
     ``last_of``: the part whose result this product is (it passes itself).  When the block
@@ -35,7 +35,7 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     such a tensor itself, whoever called it.
     """
     M, K = x.shape
-    gated = epilogue in ("gelu_tanh", "silu")
+    gated = epilogue in ("gelu_tanh", "silu", "relu")
     N, K2 = w.shape
     if gated:
         N //= 2

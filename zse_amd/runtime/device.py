@@ -162,6 +162,15 @@ KERNEL_SIGNATURES = {
     "zk_sample_cut": [_VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _I, _VP],
     "zk_penalize": [_VP, _I, _VP, _VP, _VP, _I, _VP],
     "zk_probe_read": [_VP, _SZ, _VP, _VP],
+    "zk_attention_plain_ext": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F,
+                               _I, _I, _VP, _I, _VP],
+    "zk_replicate": [_VP, _VP, _I, _I, _I, _VP],
+    "zk_streams_step": [_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _F, _VP, _VP, _I, _I, _I, _VP],
+    "zk_short_conv": [_VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _VP],
+    "zk_short_conv_state": [_VP, _VP, _I, _I, _VP, _VP, _I, _I, _I, _VP],
+    "zk_rotate_heads": [_VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
+    "zk_head_prep": [_VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_mlstm": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
@@ -249,6 +258,8 @@ class KernelLibrary:
             fn = getattr(self._dll, name)
             fn.restype, fn.argtypes = C.c_size_t, []
             setattr(self, name, fn)
+        self._dll.zk_mlstm_state_bytes.restype, self._dll.zk_mlstm_state_bytes.argtypes = C.c_size_t, [_I, _I, _I]
+        self.zk_mlstm_state_bytes = self._dll.zk_mlstm_state_bytes
         if dtype == BF16:
             self._dll.zk_attention_bf16_supports.restype = C.c_int
             self._dll.zk_attention_bf16_supports.argtypes = [_I, _I, _I, _I]
