@@ -422,8 +422,90 @@ def further_model(name, a, rt, peak_bw, peak_fl):
     return out
 
 
+# ------------------------------------------------------------------ another design beside its closest relative
+# Layer sizes that resemble real models'.  A Dafotar model here is ``groups`` times (attention with
+# a feed-forward, mLSTM without one, attention with a feed-forward that reads the first one's keys
+# and values); the Gemma 2 model beside it has as many layers of the same width, heads, head size,
+# feed-forward size, window and vocabulary.
+DESIGN_SIZES = {
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, ff=4096, groups=2, vocab=32768, window=1024),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, groups=2, vocab=32768, window=2048),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, groups=1, vocab=32768, window=4096),
+}
+
+
+def dafotar_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+           "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 2}}
+    rec = {"heads": heads, "dim": dim // 2, "vdim": dim, "gate_cap": 15.0}
+    layers = []
+    for g in range(groups):
+        layers += [{"type": "attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": ff}},
+                   {"type": "mlstm", "mixer": dict(rec), "mlp": None},
+                   {"type": "attention", "mixer": dict(att, kv_from=3 * g), "mlp": {"kind": "dense", "ff": ff}}]
+    return {"architecture": "Dafotar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": 4,
+            "canon": {"taps": 4}, "layers": layers}
+
+
+def gemma2_like(width, heads, kv_heads, dim, ff, groups, vocab, window):
+    return dict(GEMMA2_2B, num_hidden_layers=3 * groups, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=kv_heads, head_dim=dim, query_pre_attn_scalar=dim, intermediate_size=ff,
+                vocab_size=vocab, sliding_window=window, max_position_embeddings=8192)
+
+
+def state_bytes_touched(model):
+    """Bytes of per-request state a decoded token reads and writes (recurrences, convolutions)."""
+    from zse_amd.parts.base import StateNeed
+    total = sum(2 * n.nbytes for n in model.cache_needs() if isinstance(n, StateNeed))
+    for call in model.plan.order:
+        blk = model.blocks[call.layer]
+        total += sum(2 * nbytes for _, nbytes in (blk.state_needs() if hasattr(blk, "state_needs") else []))
+    return total
+
+
+def run_design(a):
+    """Prefill and decode of Dafotar beside Gemma 2 at equal layer sizes; one JSON line."""
+    from zse_amd.engine.loading import random_model
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    sizes = [s for s in a.design_sizes.split(",") if s]
+    out = {"design": "Dafotar", "beside": "Gemma 2 at equal layer sizes", "dtype": "bf16", "data": "synthetic",
+           "batch": a.batch, "context": a.context, "prefill_tokens": a.prefill_tokens, "sizes": {}}
+    for name in sizes:
+        size = DESIGN_SIZES[name]
+        rec = {"config": size}
+        for which, cfg in (("dafotar", dafotar_config(**size)), ("gemma2", gemma2_like(**size))):
+            if a.only_model and which != a.only_model:
+                continue
+            # the streams' weights near the plain residual sum, so that activations keep their size over the layers
+            model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt,
+                                 std_of={".hc": 0.3, ".temp": 0.5, "canon": 0.3})
+            tcfg = dict(cfg, vocab_size=size["vocab"])
+            t = Timed(model, rt, tcfg, a.batch, a.context, a.prefill_tokens, not a.no_graphs, page=a.page_size)
+            r = {"weights_gb": round(model.weight_bytes / 1e9, 3)}
+            if a.only != "decode":
+                pre_s, pf = t.prefill()
+                r["prefill"] = {"value": round(a.prefill_tokens / pre_s, 1), "ms": round(pre_s * 1e3, 3),
+                                "frac": round(pf / pre_s / PEAK_FLOPS["bf16"], 4)}
+            if a.only != "prefill":
+                tok_s, step_s, byts, how = t.decode(a.batch, a.steps, a.warmup)
+                byts += a.batch * state_bytes_touched(model)
+                r["decode"] = {"value": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 4), "launched": how,
+                               "roofline_frac": round(byts / step_s / PEAK_HBM, 4)}
+            log(f"{name} {which}: {r}")
+            rec[which] = r
+            t.close()
+            del t, model
+        out["sizes"][name] = rec
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=["dafotar"], default=None,
+                    help="instead of the default workload: prefill and decode of this design beside Gemma 2 at equal layer sizes")
+    ap.add_argument("--design-sizes", default="w1024,w2048,w4096", help="with --design: which of " + ", ".join(DESIGN_SIZES))
+    ap.add_argument("--only-model", choices=["dafotar", "gemma2"], default=None, help="with --design, a profiling aid: one of the two")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
@@ -452,6 +534,9 @@ def main():
         sys.exit(2)
     if a.workload:
         print(json.dumps(run_workload(a.workload, a)), flush=True)
+        return
+    if a.design:
+        run_design(a)
         return
 
     from zse_amd.engine.loading import random_model
