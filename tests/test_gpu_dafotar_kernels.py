@@ -136,6 +136,65 @@ def test_matrix_memory_cut_into_steps(dev, H, D, E):
         assert not rt.download(state)[0].any()
 
 
+@pytest.mark.parametrize("H,D,E", [(1, 8, 8), (3, 12, 20), (2, 64, 128), (1, 128, 48), (1, 256, 40)])
+def test_matrix_memory_in_chunks(dev, H, D, E):
+    """The chunked form of the recurrence with its finishing kernel: two requests side by side,
+    portions of 1 to 150 tokens (chunks of 16, 32 and 64; full, partial and single-token ones),
+    continuing from the state the portion before left."""
+    rt, k = dev
+    rng = np.random.default_rng(D + E)
+    W = 16
+    mx = {"heads": H, "dim": D, "vdim": E, "gate_cap": 5.0}
+    wts = {"q": rng.normal(size=(H * D, W)) * 0.5, "k": rng.normal(size=(H * D, W)) * 0.5,
+           "v": rng.normal(size=(H * E, W)) * 0.5, "g": rng.normal(size=(H * E, W)) * 0.5,
+           "i": rng.normal(size=(H, W)) * 2.0, "f": rng.normal(size=(H, W)) * 2.0,
+           "i.b": rng.normal(size=H), "f.b": rng.normal(size=H) + 2.0, "norm": rng.normal(1, 0.2, H * E),
+           "o": np.eye(H * E)}
+    wts = {n: a.astype(np.float32) for n, a in wts.items()}
+    lens = {0: 236, 1: 97}
+    hs = {r: rng.normal(size=(n, W)).astype(np.float32) for r, n in lens.items()}
+    want = {r: P.mlstm(h, wts, "", mx, 1e-6, np.float64) for r, h in hs.items()}
+    proj = {r: np.concatenate([h @ wts[n].T for n in ("q", "k", "v", "g")], axis=1).astype(np.float32) for r, h in hs.items()}
+    gate = {r: np.concatenate([h @ wts["i"].T, h @ wts["f"].T], axis=1).astype(np.float32) for r, h in hs.items()}
+    cuts = {0: [150, 1, 17, 64, 4], 1: [30, 33, 1, 2, 31]}
+    words = 4 + k.zk_mlstm_state_bytes(H, D, E) // 4
+    state = rt.zeros((3, words), "float32")
+    slots = [2, 0]
+    at = {0: 0, 1: 0}
+    got = {0: [], 1: []}
+    bi, bf, g = up(rt, wts["i.b"]), up(rt, wts["f.b"]), up(rt, wts["norm"])
+    for step in range(5):
+        n0, n1 = cuts[0][step], cuts[1][step]
+        T = n0 + n1
+        rows = np.concatenate([proj[0][at[0]:at[0] + n0], proj[1][at[1]:at[1] + n1]])
+        gts = np.concatenate([gate[0][at[0]:at[0] + n0], gate[1][at[1]:at[1] + n1]])
+        d_rows, d_g = up(rt, rows), up(rt, gts)
+        q_start, req = i32(rt, [0, n0, T]), i32(rt, [0] * n0 + [1] * n1)
+        d_slots = i32(rt, slots)
+        o_raw, nm, d_o = rt.zeros((T, H * E), "float32"), rt.zeros((2, H * (D + 1)), "float32"), rt.empty((T, H * E), "float32")
+        k.zk_mlstm_chunked(d_rows.ptr, rows.shape[1], d_g.ptr, bi.ptr, bf.ptr, state.ptr, words, 4, q_start.ptr, d_slots.ptr,
+                           o_raw.ptr, nm.ptr, 2, H, D, E, 5.0, max(n0, n1), rt.stream)
+        k.zk_mlstm_finish(o_raw.ptr, d_rows.ptr, rows.shape[1], g.ptr, nm.ptr, state.ptr, words, 4, req.ptr, q_start.ptr,
+                          d_slots.ptr, d_o.ptr, T, H, D, E, 1e-6, rt.stream)
+        o = rt.download(d_o)
+        got[0].append(o[:n0])
+        got[1].append(o[n0:])
+        at[0] += n0
+        at[1] += n1
+    for r in (0, 1):
+        err = np.abs(np.concatenate(got[r]) - want[r]).max()
+        assert err < 5e-5 * max(1.0, np.abs(want[r]).max()), (r, err)
+    # and the state it leaves is the one the token-by-token kernel leaves
+    seq = rt.zeros((3, words), "float32")
+    for r in (0, 1):
+        d_o = rt.empty((lens[r], H * E), "float32")
+        k.zk_mlstm(up(rt, proj[r]).ptr, proj[r].shape[1], up(rt, gate[r]).ptr, bi.ptr, bf.ptr, g.ptr, seq.ptr, words, 4,
+                   i32(rt, [0, lens[r]]).ptr, i32(rt, [slots[r]]).ptr, d_o.ptr, 1, H, D, E, 5.0, 1e-6, rt.stream)
+    a, b = rt.download(state), rt.download(seq)
+    assert np.abs(a - b).max() < 1e-4 * max(1.0, np.abs(b).max())
+    assert not a[1].any() and not a[:, :4].any()
+
+
 def test_the_running_maximum_starts_at_zero(dev):
     """With strongly negative input gates the first outputs are governed by exp(-m) with m = 0
     in the denominator; a maximum that started at minus infinity would give other values."""

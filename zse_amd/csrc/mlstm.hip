@@ -104,6 +104,263 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
   if (tid == 0) st[(size_t)D * E + D] = m;
 }
 
+// ---- the same recurrence over chunks of L tokens, for steps that bring portions of prompts.
+//
+// Inside a chunk that starts from the state (S0, n0, m0), with F_j the sum of the forget gates up
+// to token j of the chunk and a_s = i_s - F_s:
+//
+//   M_j = max(m0, max_{s<=j} a_s)                     m_j = F_j + M_j
+//   P_js = (q_j . k_s) exp(a_s - M_j)  for s <= j     g_j = exp(m0 - M_j)
+//   S_j^T q_j = g_j S0^T q_j + sum_s P_js v_s         n_j . q_j = g_j n0 . q_j + sum_s P_js
+//
+// which is the token-by-token recurrence written out (every exponent is <= 0).  At the chunk's
+// last token the state becomes g S0 + sum_s exp(a_s - M) k_s v_s^T.  So a chunk is four small
+// matrix products (q k^T, P v, q S0, k^T v) instead of L dependent steps.  A block owns 32
+// value channels of a head: the recurrence never mixes value channels, only the norm over a
+// head's read-out does, and that (with the gain and the output gate) is left to a second
+// kernel, which also stores the new n and m: every block of a head computes them, none may
+// store them while another still reads the old ones.
+#define MLSTM_EC 32
+
+template <int L>
+__global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
+    const act_t* __restrict__ qkvz, int ld, const float* __restrict__ gates, const float* __restrict__ bias_i,
+    const float* __restrict__ bias_f, float* __restrict__ state, int slot_words, int offset_words,
+    const int* __restrict__ q_start, const int* __restrict__ slot_of_req, float* __restrict__ o_raw,
+    float* __restrict__ nm_new, int H, int D, int E, float cap, float q_scale) {
+  constexpr int EC = MLSTM_EC;
+  constexpr int TP = L / 16;
+  extern __shared__ float lds[];
+  const int r = blockIdx.x, hd = blockIdx.y, e0 = blockIdx.z * EC, tid = threadIdx.x;
+  const int t0 = q_start[r], t1 = q_start[r + 1];
+  if (t1 <= t0) return;
+  const int DP = D + 1, LP = L + 1;
+  float* Ss = lds;                      // [D][EC]   this block's columns of S
+  float* ns = Ss + (size_t)D * EC;      // [D]
+  float* Qs = ns + D;                   // [L][DP]
+  float* Ks = Qs + (size_t)L * DP;      // [L][DP]
+  float* Vs = Ks + (size_t)L * DP;      // [L][EC]
+  float* Ps = Vs + (size_t)L * EC;      // [L][LP]
+  float* ga = Ps + (size_t)L * LP;      // a_s, then (after the scan) i_s - F_s
+  float* gM = ga + L;                   // M_j
+  float* gF = gM + L;                   // f_s, then F_j
+  float* gden = gF + L;                 // denominators
+  float* gw = gden + L;                 // exp(a_s - M_last)
+  const size_t per_head = (size_t)D * E + D + 1;
+  float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * per_head;
+  for (int i = tid; i < D * EC; i += MLSTM_THREADS) {
+    const int d = i / EC, e = e0 + i % EC;
+    Ss[i] = e < E ? st[(size_t)d * E + e] : 0.f;
+  }
+  for (int d = tid; d < D; d += MLSTM_THREADS) ns[d] = st[(size_t)D * E + d];
+  float m_prev = st[(size_t)D * E + D];
+  const float bi = bias_i[hd], bf = bias_f[hd];
+  __syncthreads();
+  for (int c0 = t0; c0 < t1; c0 += L) {
+    const int Lc = min(L, t1 - c0);
+    for (int i = tid; i < L * D; i += MLSTM_THREADS) {
+      const int j = i / D, d = i % D;
+      float q = 0.f, k = 0.f;
+      if (j < Lc) {
+        const act_t* row = qkvz + (size_t)(c0 + j) * ld;
+        q = to_f32(row[(size_t)hd * D + d]) * q_scale;
+        k = to_f32(row[(size_t)(H + hd) * D + d]);
+      }
+      Qs[j * DP + d] = q;
+      Ks[j * DP + d] = k;
+    }
+    for (int i = tid; i < L * EC; i += MLSTM_THREADS) {
+      const int j = i / EC, e = e0 + i % EC;
+      Vs[i] = (j < Lc && e < E) ? to_f32(qkvz[(size_t)(c0 + j) * ld + (size_t)2 * H * D + (size_t)hd * E + e]) : 0.f;
+    }
+    if (tid < Lc) {
+      const size_t t = c0 + tid;
+      ga[tid] = cap * tanhf((gates[t * 2 * H + hd] + bi) / cap);
+      gF[tid] = log_sigmoid(cap * tanhf((gates[t * 2 * H + H + hd] + bf) / cap));
+    }
+    __syncthreads();
+    if (tid == 0) {
+      float F = 0.f, M = m_prev;
+      for (int j = 0; j < L; j++) {
+        if (j < Lc) {
+          F += gF[j];
+          const float a = ga[j] - F;
+          M = fmaxf(M, a);
+          ga[j] = a;
+        } else {
+          ga[j] = -INFINITY;
+        }
+        gM[j] = M;
+        gF[j] = F;
+      }
+    }
+    __syncthreads();
+    {  // P
+      const int pj = (tid / 16) * TP, ps = (tid % 16) * TP;
+      float acc[TP][TP] = {};
+      for (int d = 0; d < D; d++) {
+        float q[TP], k[TP];
+#pragma unroll
+        for (int x = 0; x < TP; x++) {
+          q[x] = Qs[(pj + x) * DP + d];
+          k[x] = Ks[(ps + x) * DP + d];
+        }
+#pragma unroll
+        for (int a = 0; a < TP; a++)
+#pragma unroll
+          for (int b = 0; b < TP; b++) acc[a][b] = fmaf(q[a], k[b], acc[a][b]);
+      }
+#pragma unroll
+      for (int a = 0; a < TP; a++)
+#pragma unroll
+        for (int b = 0; b < TP; b++) {
+          const int j = pj + a, s2 = ps + b;
+          Ps[j * LP + s2] = (s2 <= j && j < Lc) ? acc[a][b] * expf(ga[s2] - gM[j]) : 0.f;
+        }
+    }
+    __syncthreads();
+    if (tid < L) {  // denominators
+      const int j = tid;
+      float nq = 0.f;
+      for (int d = 0; d < D; d++) nq = fmaf(ns[d], Qs[j * DP + d], nq);
+      nq *= expf(m_prev - gM[j]);
+      for (int s2 = 0; s2 <= j; s2++) nq += Ps[j * LP + s2];
+      gden[j] = fmaxf(fabsf(nq), expf(-(gF[j] + gM[j]))) + 1e-6f;
+      gw[j] = j < Lc ? expf(ga[j] - gM[Lc - 1]) : 0.f;
+    }
+    {  // read-out: rows rg .. rg + TP - 1, columns ec, ec + 1
+      const int ec = (tid % 16) * 2, rg = (tid / 16) * TP;
+      float acc[TP][2] = {};
+      for (int d = 0; d < D; d++) {
+        const float s0 = Ss[d * EC + ec], s1 = Ss[d * EC + ec + 1];
+#pragma unroll
+        for (int a = 0; a < TP; a++) {
+          const float q = Qs[(rg + a) * DP + d];
+          acc[a][0] = fmaf(q, s0, acc[a][0]);
+          acc[a][1] = fmaf(q, s1, acc[a][1]);
+        }
+      }
+#pragma unroll
+      for (int a = 0; a < TP; a++) {
+        const float g = expf(m_prev - gM[rg + a]);
+        acc[a][0] *= g;
+        acc[a][1] *= g;
+      }
+      for (int s2 = 0; s2 < Lc; s2++) {
+        const float v0 = Vs[s2 * EC + ec], v1 = Vs[s2 * EC + ec + 1];
+#pragma unroll
+        for (int a = 0; a < TP; a++) {
+          const float p = Ps[(rg + a) * LP + s2];
+          acc[a][0] = fmaf(p, v0, acc[a][0]);
+          acc[a][1] = fmaf(p, v1, acc[a][1]);
+        }
+      }
+      __syncthreads();          // the denominators are there; every read of Vs is done
+#pragma unroll
+      for (int a = 0; a < TP; a++) {
+        const int j = rg + a;
+        if (j < Lc) {
+          float* o = o_raw + ((size_t)(c0 + j) * H + hd) * E;
+          if (e0 + ec < E) o[e0 + ec] = acc[a][0] / gden[j];
+          if (e0 + ec + 1 < E) o[e0 + ec + 1] = acc[a][1] / gden[j];
+        }
+      }
+    }
+    // the state after the chunk's last token
+    const float M_last = gM[Lc - 1];
+    const float g_last = expf(m_prev - M_last);
+    const float m_next = gF[Lc - 1] + M_last;
+    for (int i = tid; i < L * EC; i += MLSTM_THREADS) Vs[i] *= gw[i / EC];
+    for (int d = tid; d < D; d += MLSTM_THREADS) {
+      float acc = 0.f;
+      for (int s2 = 0; s2 < Lc; s2++) acc = fmaf(gw[s2], Ks[s2 * DP + d], acc);
+      ns[d] = fmaf(g_last, ns[d], acc);
+    }
+    __syncthreads();
+    {
+      const int ec = (tid % 16) * 2, dg = (tid / 16) * 4;
+      for (int db = 0; db < D; db += 64) {
+        float acc[4][2] = {};
+        const int d = db + dg;
+        for (int s2 = 0; s2 < Lc; s2++) {
+          const float v0 = Vs[s2 * EC + ec], v1 = Vs[s2 * EC + ec + 1];
+#pragma unroll
+          for (int a = 0; a < 4; a++) {
+            const float k = d + a < D ? Ks[s2 * DP + d + a] : 0.f;
+            acc[a][0] = fmaf(k, v0, acc[a][0]);
+            acc[a][1] = fmaf(k, v1, acc[a][1]);
+          }
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+          if (d + a < D) {
+            float* sp = Ss + (size_t)(d + a) * EC + ec;
+            sp[0] = fmaf(g_last, sp[0], acc[a][0]);
+            sp[1] = fmaf(g_last, sp[1], acc[a][1]);
+          }
+      }
+    }
+    m_prev = m_next;
+    __syncthreads();
+  }
+  for (int i = tid; i < D * EC; i += MLSTM_THREADS) {
+    const int d = i / EC, e = e0 + i % EC;
+    if (e < E) st[(size_t)d * E + e] = Ss[i];
+  }
+  if (blockIdx.z == 0) {
+    float* nm = nm_new + ((size_t)r * H + hd) * (D + 1);
+    for (int d = tid; d < D; d += MLSTM_THREADS) nm[d] = ns[d];
+    if (tid == 0) nm[D] = m_prev;
+  }
+}
+
+// The read-out's norm over each head, gain and output gate; the block of a request's last
+// token also stores the head's new n and m.
+__global__ __launch_bounds__(64) void mlstm_finish_kernel(
+    const float* __restrict__ o_raw, const act_t* __restrict__ qkvz, int ld, const float* __restrict__ norm_w,
+    const float* __restrict__ nm_new, float* __restrict__ state, int slot_words, int offset_words,
+    const int* __restrict__ req_of_token, const int* __restrict__ q_start, const int* __restrict__ slot_of_req,
+    act_t* __restrict__ out, int H, int D, int E, float eps) {
+  const int t = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x;
+  const float* o = o_raw + ((size_t)t * H + hd) * E;
+  float ss = 0.f;
+  for (int e = lane; e < E; e += 64) ss = fmaf(o[e], o[e], ss);
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)E + eps);
+  const act_t* z = qkvz + (size_t)t * ld + (size_t)2 * H * D + (size_t)H * E + (size_t)hd * E;
+  for (int e = lane; e < E; e += 64) {
+    const float y = o[e] * inv * norm_w[(size_t)hd * E + e] * (1.0f / (1.0f + expf(-to_f32(z[e]))));
+    out[((size_t)t * H + hd) * E + e] = from_f32<act_t>(y);
+  }
+  const int r = req_of_token[t];
+  if (t == q_start[r + 1] - 1) {
+    float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * ((size_t)D * E + D + 1) + (size_t)D * E;
+    const float* nm = nm_new + ((size_t)r * H + hd) * (D + 1);
+    for (int d = lane; d <= D; d += 64) st[d] = nm[d];
+  }
+}
+
+static size_t mlstm_chunk_lds(int L, int D) {
+  return ((size_t)D * MLSTM_EC + D + (size_t)2 * L * (D + 1) + (size_t)L * MLSTM_EC + (size_t)L * (L + 1) + 5 * L + 8) * 4;
+}
+
+template <int L>
+static int mlstm_chunk_launch(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+                              float* state, int slot_words, int offset_words, const int* q_start,
+                              const int* slot_of_req, float* o_raw, float* nm_new, int R, int H, int D, int E,
+                              float cap, hipStream_t stream) {
+  const size_t lds = mlstm_chunk_lds(L, D);
+  static size_t raised = 0;
+  if (lds > 48 * 1024 && lds > raised) {
+    hipFuncSetAttribute((const void*)mlstm_chunk_kernel<L>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    raised = lds;
+  }
+  dim3 grid(R, H, (E + MLSTM_EC - 1) / MLSTM_EC);
+  mlstm_chunk_kernel<L><<<grid, MLSTM_THREADS, lds, stream>>>((const act_t*)qkvz, ld, gates, bias_i, bias_f, state,
+                                                              slot_words, offset_words, q_start, slot_of_req, o_raw,
+                                                              nm_new, H, D, E, cap, 1.0f / sqrtf((float)D));
+  return zk_launch_status("zk_mlstm_chunked");
+}
+
 extern "C" {
 
 size_t zk_mlstm_state_bytes(int H, int D, int E) { return (size_t)H * ((size_t)D * E + D + 1) * 4; }
@@ -136,6 +393,43 @@ int zk_mlstm(const void* qkvz, int ld, const float* gates, const float* bias_i, 
   return zk_launch_status("zk_mlstm");
 }
 
+// The same as zk_mlstm for steps that bring portions: chunks of up to 64 tokens (fewer where
+// max_q_len, the longest portion of the step, or the local memory asks for less).  o_raw: float
+// [T, H * E] scratch; nm_new: float [R, H, D + 1] scratch.  zk_mlstm_finish must follow.
+int zk_mlstm_chunked(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+                     float* state, int slot_words, int offset_words, const int* q_start, const int* slot_of_req,
+                     float* o_raw, float* nm_new, int R, int H, int D, int E, float cap, int max_q_len, void* stream) {
+  ZK_REQUIRE(R >= 0 && R <= 65535 && H > 0 && H <= 65535 && D > 0 && E > 0, "zk_mlstm_chunked: bad sizes");
+  ZK_REQUIRE(D <= 256 && E <= 2048, "zk_mlstm_chunked: heads of more than 256 key channels are not supported");
+  ZK_REQUIRE(ld >= 2 * H * (D + E), "zk_mlstm_chunked: rows too short");
+  ZK_REQUIRE(cap > 0.f, "zk_mlstm_chunked: the gates' cap must be positive");
+  ZK_REQUIRE((size_t)slot_words * 4 >= (size_t)offset_words * 4 + zk_mlstm_state_bytes(H, D, E),
+             "zk_mlstm_chunked: the state does not fit its slot");
+  if (R == 0) return 0;
+  int L = max_q_len <= 16 ? 16 : max_q_len <= 32 ? 32 : 64;
+  while (L > 16 && mlstm_chunk_lds(L, D) > 150 * 1024) L /= 2;
+  hipStream_t s = (hipStream_t)stream;
+#define ZK_CHUNK_(L_) \
+  mlstm_chunk_launch<L_>(qkvz, ld, gates, bias_i, bias_f, state, slot_words, offset_words, q_start, slot_of_req, o_raw, \
+                         nm_new, R, H, D, E, cap, s)
+  return L == 64 ? ZK_CHUNK_(64) : L == 32 ? ZK_CHUNK_(32) : ZK_CHUNK_(16);
+#undef ZK_CHUNK_
+}
+
+int zk_mlstm_finish(const float* o_raw, const void* qkvz, int ld, const float* norm_w, const float* nm_new,
+                    float* state, int slot_words, int offset_words, const int* req_of_token, const int* q_start,
+                    const int* slot_of_req, void* out, int T, int H, int D, int E, float eps, void* stream) {
+  ZK_REQUIRE(T >= 0 && H > 0 && H <= 65535 && D > 0 && E > 0, "zk_mlstm_finish: bad sizes");
+  if (T == 0) return 0;
+  dim3 grid(T, H);
+  mlstm_finish_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(o_raw, (const act_t*)qkvz, ld, norm_w, nm_new, state,
+                                                            slot_words, offset_words, req_of_token, q_start, slot_of_req,
+                                                            (act_t*)out, H, D, E, eps);
+  return zk_launch_status("zk_mlstm_finish");
+}
+
 }  // extern "C"
 
 ZK_ENTER(zk_mlstm)
+ZK_ENTER(zk_mlstm_chunked)
+ZK_ENTER(zk_mlstm_finish)

@@ -10,12 +10,15 @@ at zero and is carried as floats in the request's state slot:
     out = W_o ( o_t / sqrt(mean(o_t^2) + eps) * g * sigmoid(W_z x_t) )      (the mean per head)
 
 q, k, v and z are one product; the two gates are a second, small one whose results stay float.
+Steps of single tokens run the recurrence as written, one block per (request, head); steps with
+portions of prompts run it over chunks of up to 64 tokens, where it becomes four small matrix
+products per chunk, with a head's value channels spread over several blocks.
 """
 from __future__ import annotations
 
 from typing import List
 
-from ..runtime.device import F32, Tensor
+from ..runtime.device import BF16, F32, Tensor
 from .base import ROLE_GAIN, Part, StateNeed, TensorReq, register_part
 from .ops import linear
 
@@ -67,9 +70,21 @@ class MatrixMemory(Part):
         qkvz = linear(ctx, x, self.w_qkvz, ctx.alloc((T, ld)))
         gates = linear(ctx, x, self.w_gates, ctx.alloc((T, 2 * H), F32))
         out = ctx.alloc((T, H * E))
-        k.zk_mlstm(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, self.gain.ptr, ctx.state.ptr,
-                   ctx.state.shape[1], cache.state_offset // 4, ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, D, E,
-                   float(s.gate_cap), float(s.eps), ctx.stream)
+        words, at = ctx.state.shape[1], cache.state_offset // 4
+        if ctx.max_q_len > 1 and ctx.dtype == BF16 and D <= 256:
+            # a step with portions of prompts: chunks of tokens as small matrix products, then the
+            # heads' norm and gate.  (In 32-bit every step runs token by token, so that a request's
+            # values are the same bits however its tokens are cut into steps.)
+            o_raw = ctx.alloc((T, H * E), F32)
+            nm = ctx.alloc((ctx.R, H * (D + 1)), F32)
+            k.zk_mlstm_chunked(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, ctx.state.ptr, words, at,
+                               ctx.q_start, ctx.slot_of_req, o_raw.ptr, nm.ptr, ctx.R, H, D, E, float(s.gate_cap),
+                               int(ctx.max_q_len), ctx.stream)
+            k.zk_mlstm_finish(o_raw.ptr, qkvz.ptr, ld, self.gain.ptr, nm.ptr, ctx.state.ptr, words, at, ctx.req_of_token,
+                              ctx.q_start, ctx.slot_of_req, out.ptr, T, H, D, E, float(s.eps), ctx.stream)
+        else:
+            k.zk_mlstm(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, self.gain.ptr, ctx.state.ptr, words, at,
+                       ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, D, E, float(s.gate_cap), float(s.eps), ctx.stream)
         return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 

@@ -171,6 +171,8 @@ KERNEL_SIGNATURES = {
     "zk_rotate_heads": [_VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
     "zk_head_prep": [_VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
     "zk_mlstm": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
+    "zk_mlstm_chunked": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
+    "zk_mlstm_finish": [_VP, _VP, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
