@@ -26,6 +26,11 @@ __device__ __forceinline__ float log_sigmoid(float x) {
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
+// DIRECT: S stays in the state slot and every element is read, renewed and written back once per
+// token, many loads in flight (steps of single tokens, where staging S through the local memory
+// would only add two passes); else S is staged for the step's tokens.  The same arithmetic in
+// the same order either way.
+template <bool DIRECT>
 __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
     const act_t* __restrict__ qkvz, int ld, const float* __restrict__ gates, const float* __restrict__ bias_i,
     const float* __restrict__ bias_f, const float* __restrict__ norm_w, float* __restrict__ state, int slot_words,
@@ -35,16 +40,20 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
   const int r = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x;
   const int t0 = q_start[r], t1 = q_start[r + 1];
   if (t1 <= t0) return;                       // a padding request of a captured step
-  float* S = lds;                              // [D][E]
-  float* n = S + (size_t)D * E;                // [D]
+  const size_t per_head = (size_t)D * E + D + 1;
+  float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * per_head;
+  float* S = DIRECT ? st : lds;                // [D][E]
+  float* n = DIRECT ? lds : lds + (size_t)D * E;      // [D]
   float* sq = n + D;                           // [D]
   float* sk = sq + D;                          // [D]
   float* sv = sk + D;                          // [E]
   float* part = sv + E;                        // [slices][E]
   float* red = part + MLSTM_THREADS;           // 17 + 1
-  const size_t per_head = (size_t)D * E + D + 1;
-  float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * per_head;
-  for (int i = tid; i < D * E + D; i += MLSTM_THREADS) lds[i] = st[i];
+  if (DIRECT) {
+    for (int d = tid; d < D; d += MLSTM_THREADS) n[d] = st[(size_t)D * E + d];
+  } else {
+    for (int i = tid; i < D * E + D; i += MLSTM_THREADS) lds[i] = st[i];
+  }
   float m = st[(size_t)D * E + D];
   const int slices = MLSTM_THREADS / E > 0 ? MLSTM_THREADS / E : 1;     // E <= 256
   const int e = tid % E, sl = tid / E;
@@ -100,7 +109,11 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
     }
     __syncthreads();
   }
-  for (int i = tid; i < D * E + D; i += MLSTM_THREADS) st[i] = lds[i];
+  if (DIRECT) {
+    for (int d = tid; d < D; d += MLSTM_THREADS) st[(size_t)D * E + d] = n[d];
+  } else {
+    for (int i = tid; i < D * E + D; i += MLSTM_THREADS) st[i] = lds[i];
+  }
   if (tid == 0) st[(size_t)D * E + D] = m;
 }
 
@@ -121,6 +134,17 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
 // kernel, which also stores the new n and m: every block of a head computes them, none may
 // store them while another still reads the old ones.
 #define MLSTM_EC 32
+
+__device__ __forceinline__ void load8(const float* p, float v[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const __bf16* p, float v[8]) {
+  typedef __bf16 bf8 __attribute__((ext_vector_type(8)));
+  const bf8 a = *(const bf8*)p;
+#pragma unroll
+  for (int x = 0; x < 8; x++) v[x] = (float)a[x];
+}
 
 template <int L>
 __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
@@ -155,19 +179,38 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
   for (int d = tid; d < D; d += MLSTM_THREADS) ns[d] = st[(size_t)D * E + d];
   float m_prev = st[(size_t)D * E + D];
   const float bi = bias_i[hd], bf = bias_f[hd];
+  const bool vec8 = D % 8 == 0 && ld % 8 == 0 && (uintptr_t)qkvz % 16 == 0;
   __syncthreads();
   for (int c0 = t0; c0 < t1; c0 += L) {
     const int Lc = min(L, t1 - c0);
-    for (int i = tid; i < L * D; i += MLSTM_THREADS) {
-      const int j = i / D, d = i % D;
-      float q = 0.f, k = 0.f;
-      if (j < Lc) {
-        const act_t* row = qkvz + (size_t)(c0 + j) * ld;
-        q = to_f32(row[(size_t)hd * D + d]) * q_scale;
-        k = to_f32(row[(size_t)(H + hd) * D + d]);
+    if (vec8) {      // eight channels a load
+      const int D8 = D / 8;
+      for (int i = tid; i < L * D8; i += MLSTM_THREADS) {
+        const int j = i / D8, d = (i % D8) * 8;
+        float q[8] = {}, k[8] = {};
+        if (j < Lc) {
+          const act_t* row = qkvz + (size_t)(c0 + j) * ld;
+          load8(row + (size_t)hd * D + d, q);
+          load8(row + (size_t)(H + hd) * D + d, k);
+        }
+#pragma unroll
+        for (int x = 0; x < 8; x++) {
+          Qs[j * DP + d + x] = q[x] * q_scale;
+          Ks[j * DP + d + x] = k[x];
+        }
       }
-      Qs[j * DP + d] = q;
-      Ks[j * DP + d] = k;
+    } else {
+      for (int i = tid; i < L * D; i += MLSTM_THREADS) {
+        const int j = i / D, d = i % D;
+        float q = 0.f, k = 0.f;
+        if (j < Lc) {
+          const act_t* row = qkvz + (size_t)(c0 + j) * ld;
+          q = to_f32(row[(size_t)hd * D + d]) * q_scale;
+          k = to_f32(row[(size_t)(H + hd) * D + d]);
+        }
+        Qs[j * DP + d] = q;
+        Ks[j * DP + d] = k;
+      }
     }
     for (int i = tid; i < L * EC; i += MLSTM_THREADS) {
       const int j = i / EC, e = e0 + i % EC;
@@ -179,31 +222,38 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
       gF[tid] = log_sigmoid(cap * tanhf((gates[t * 2 * H + H + hd] + bf) / cap));
     }
     __syncthreads();
-    if (tid == 0) {
-      float F = 0.f, M = m_prev;
-      for (int j = 0; j < L; j++) {
-        if (j < Lc) {
-          F += gF[j];
-          const float a = ga[j] - F;
-          M = fmaxf(M, a);
-          ga[j] = a;
-        } else {
-          ga[j] = -INFINITY;
-        }
-        gM[j] = M;
+    if (tid < ZSE_WAVE) {      // running sums of the forget gates and running maxima of a, over one wave (L <= 64)
+      const int j = tid;
+      float F = j < Lc ? gF[j] : 0.f;
+#pragma unroll
+      for (int o = 1; o < ZSE_WAVE; o <<= 1) {
+        const float up = __shfl_up(F, o, ZSE_WAVE);
+        if (j >= o) F += up;
+      }
+      const float a = j < Lc ? ga[j] - F : -INFINITY;
+      float M = a;
+#pragma unroll
+      for (int o = 1; o < ZSE_WAVE; o <<= 1) {
+        const float up = __shfl_up(M, o, ZSE_WAVE);
+        if (j >= o) M = fmaxf(M, up);
+      }
+      if (j < L) {
+        ga[j] = a;
+        gM[j] = fmaxf(M, m_prev);
         gF[j] = F;
       }
     }
     __syncthreads();
     {  // P
-      const int pj = (tid / 16) * TP, ps = (tid % 16) * TP;
+      // rows pj + 16 a, columns ps + 16 b: neighbouring lanes read neighbouring rows of K
+      const int pj = tid / 16, ps = tid % 16;
       float acc[TP][TP] = {};
       for (int d = 0; d < D; d++) {
         float q[TP], k[TP];
 #pragma unroll
         for (int x = 0; x < TP; x++) {
-          q[x] = Qs[(pj + x) * DP + d];
-          k[x] = Ks[(ps + x) * DP + d];
+          q[x] = Qs[(pj + 16 * x) * DP + d];
+          k[x] = Ks[(ps + 16 * x) * DP + d];
         }
 #pragma unroll
         for (int a = 0; a < TP; a++)
@@ -214,7 +264,7 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
       for (int a = 0; a < TP; a++)
 #pragma unroll
         for (int b = 0; b < TP; b++) {
-          const int j = pj + a, s2 = ps + b;
+          const int j = pj + 16 * a, s2 = ps + 16 * b;
           Ps[j * LP + s2] = (s2 <= j && j < Lc) ? acc[a][b] * expf(ga[s2] - gM[j]) : 0.f;
         }
     }
@@ -228,21 +278,21 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
       gden[j] = fmaxf(fabsf(nq), expf(-(gF[j] + gM[j]))) + 1e-6f;
       gw[j] = j < Lc ? expf(ga[j] - gM[Lc - 1]) : 0.f;
     }
-    {  // read-out: rows rg .. rg + TP - 1, columns ec, ec + 1
-      const int ec = (tid % 16) * 2, rg = (tid / 16) * TP;
+    {  // read-out: TP rows, columns ec, ec + 1
+      const int ec = (tid % 16) * 2, rg = tid / 16;        // rows rg + 16 a
       float acc[TP][2] = {};
       for (int d = 0; d < D; d++) {
         const float s0 = Ss[d * EC + ec], s1 = Ss[d * EC + ec + 1];
 #pragma unroll
         for (int a = 0; a < TP; a++) {
-          const float q = Qs[(rg + a) * DP + d];
+          const float q = Qs[(rg + 16 * a) * DP + d];
           acc[a][0] = fmaf(q, s0, acc[a][0]);
           acc[a][1] = fmaf(q, s1, acc[a][1]);
         }
       }
 #pragma unroll
       for (int a = 0; a < TP; a++) {
-        const float g = expf(m_prev - gM[rg + a]);
+        const float g = expf(m_prev - gM[rg + 16 * a]);
         acc[a][0] *= g;
         acc[a][1] *= g;
       }
@@ -250,7 +300,7 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
         const float v0 = Vs[s2 * EC + ec], v1 = Vs[s2 * EC + ec + 1];
 #pragma unroll
         for (int a = 0; a < TP; a++) {
-          const float p = Ps[(rg + a) * LP + s2];
+          const float p = Ps[(rg + 16 * a) * LP + s2];
           acc[a][0] = fmaf(p, v0, acc[a][0]);
           acc[a][1] = fmaf(p, v1, acc[a][1]);
         }
@@ -258,7 +308,7 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_chunk_kernel(
       __syncthreads();          // the denominators are there; every read of Vs is done
 #pragma unroll
       for (int a = 0; a < TP; a++) {
-        const int j = rg + a;
+        const int j = rg + 16 * a;
         if (j < Lc) {
           float* o = o_raw + ((size_t)(c0 + j) * H + hd) * E;
           if (e0 + ec < E) o[e0 + ec] = acc[a][0] / gden[j];
@@ -367,9 +417,9 @@ size_t zk_mlstm_state_bytes(int H, int D, int E) { return (size_t)H * ((size_t)D
 
 // qkvz: [T, ld] activations, a row holding q [H, D] | k [H, D] | v [H, E] | z [H, E];
 // gates: float [T, 2H] (input gates, then forget gates, before bias and cap); out: [T, H * E].
-int zk_mlstm(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
-             const float* norm_w, float* state, int slot_words, int offset_words, const int* q_start,
-             const int* slot_of_req, void* out, int R, int H, int D, int E, float cap, float eps, void* stream) {
+static int mlstm_run(bool direct, const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+                     const float* norm_w, float* state, int slot_words, int offset_words, const int* q_start,
+                     const int* slot_of_req, void* out, int R, int H, int D, int E, float cap, float eps, void* stream) {
   ZK_REQUIRE(R >= 0 && H > 0 && H <= 65535 && D > 0 && E > 0, "zk_mlstm: bad sizes");
   ZK_REQUIRE(E <= MLSTM_THREADS, "zk_mlstm: more than 256 value channels a head are not supported");
   ZK_REQUIRE(ld >= 2 * H * (D + E), "zk_mlstm: rows too short");
@@ -377,20 +427,41 @@ int zk_mlstm(const void* qkvz, int ld, const float* gates, const float* bias_i, 
   ZK_REQUIRE((size_t)slot_words * 4 >= (size_t)offset_words * 4 + zk_mlstm_state_bytes(H, D, E),
              "zk_mlstm: the state does not fit its slot");
   if (R == 0) return 0;
-  const size_t lds = ((size_t)D * E + 3 * D + E + MLSTM_THREADS + 32) * 4;
+  const size_t lds = ((direct ? 0 : (size_t)D * E) + 3 * D + E + MLSTM_THREADS + 32) * 4;
   ZK_REQUIRE(lds <= 160 * 1024, "zk_mlstm: a head's state does not fit the local memory");
   if (lds > 48 * 1024) {
     static size_t raised = 0;
     if (lds > raised) {
-      hipFuncSetAttribute((const void*)mlstm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      hipFuncSetAttribute((const void*)mlstm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       raised = lds;
     }
   }
   dim3 grid(R, H);
-  mlstm_kernel<<<grid, MLSTM_THREADS, lds, (hipStream_t)stream>>>(
-      (const act_t*)qkvz, ld, gates, bias_i, bias_f, norm_w, state, slot_words, offset_words, q_start, slot_of_req,
-      (act_t*)out, H, D, E, cap, eps, 1.0f / sqrtf((float)D));
+  if (direct)
+    mlstm_kernel<true><<<grid, MLSTM_THREADS, lds, (hipStream_t)stream>>>(
+        (const act_t*)qkvz, ld, gates, bias_i, bias_f, norm_w, state, slot_words, offset_words, q_start, slot_of_req,
+        (act_t*)out, H, D, E, cap, eps, 1.0f / sqrtf((float)D));
+  else
+    mlstm_kernel<false><<<grid, MLSTM_THREADS, lds, (hipStream_t)stream>>>(
+        (const act_t*)qkvz, ld, gates, bias_i, bias_f, norm_w, state, slot_words, offset_words, q_start, slot_of_req,
+        (act_t*)out, H, D, E, cap, eps, 1.0f / sqrtf((float)D));
   return zk_launch_status("zk_mlstm");
+}
+
+int zk_mlstm(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+             const float* norm_w, float* state, int slot_words, int offset_words, const int* q_start,
+             const int* slot_of_req, void* out, int R, int H, int D, int E, float cap, float eps, void* stream) {
+  return mlstm_run(false, qkvz, ld, gates, bias_i, bias_f, norm_w, state, slot_words, offset_words, q_start, slot_of_req,
+                   out, R, H, D, E, cap, eps, stream);
+}
+
+// The same for steps in which every request brings one token: the state is renewed where it lies.
+// (Right for any step, and bit for bit what zk_mlstm gives; only slower where requests bring more.)
+int zk_mlstm_token(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+                   const float* norm_w, float* state, int slot_words, int offset_words, const int* q_start,
+                   const int* slot_of_req, void* out, int R, int H, int D, int E, float cap, float eps, void* stream) {
+  return mlstm_run(true, qkvz, ld, gates, bias_i, bias_f, norm_w, state, slot_words, offset_words, q_start, slot_of_req,
+                   out, R, H, D, E, cap, eps, stream);
 }
 
 // The same as zk_mlstm for steps that bring portions: chunks of up to 64 tokens (fewer where
@@ -431,5 +502,6 @@ int zk_mlstm_finish(const float* o_raw, const void* qkvz, int ld, const float* n
 }  // extern "C"
 
 ZK_ENTER(zk_mlstm)
+ZK_ENTER(zk_mlstm_token)
 ZK_ENTER(zk_mlstm_chunked)
 ZK_ENTER(zk_mlstm_finish)

@@ -33,7 +33,10 @@ __global__ void replicate_kernel(const float* __restrict__ src, float* __restric
   }
 }
 
-__global__ __launch_bounds__(256) void streams_step_kernel(
+// V channels a thread and pass (4 where rows are whole 16-byte pieces, else 1); the block is 256
+// threads wide, or 1,024 for steps of few rows, which are bound by the latency of their loads.
+template <int V>
+__global__ __launch_bounds__(1024) void streams_step_kernel(
     float* __restrict__ xs, int S, const void* __restrict__ y, int y_parts, size_t y_plane,
     const float* __restrict__ w_mix, const float* __restrict__ w_out, const float* __restrict__ w_in,
     const float* __restrict__ norm_w, const float* __restrict__ norm_b, float eps, const int* __restrict__ rows,
@@ -41,7 +44,7 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
   extern __shared__ float u_row[];          // W floats
   __shared__ float s_mix[STREAMS_MAX * STREAMS_MAX], s_out[STREAMS_MAX], s_in[STREAMS_MAX];
   __shared__ float scratch[17];
-  const int b = blockIdx.x, tid = threadIdx.x;
+  const int b = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
   const int t = rows ? rows[b] : b;
   if (tid < S * S && w_mix) s_mix[tid] = w_mix[tid];
   if (tid < S) {
@@ -51,62 +54,87 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
   __syncthreads();
   float* x = xs + (size_t)t * S * W;
   float sum = 0.f;
-  for (int c = tid; c < W; c += 256) {
-    float v[STREAMS_MAX];
+  for (int c = tid * V; c < W; c += nt * V) {
+    float v[STREAMS_MAX][V];
 #pragma unroll
-    for (int s = 0; s < STREAMS_MAX; s++) v[s] = s < S ? x[(size_t)s * W + c] : 0.f;
-    if (y != nullptr) {
-      float yv;
-      if (y_parts > 0) {      // planes of a product that split K: added in order, rounded as the join would
-        const float* p = (const float*)y + (size_t)t * W + c;
-        yv = p[0];
-        for (int k = 1; k < y_parts; k++) yv += p[k * y_plane];
-        yv = to_f32(from_f32<act_t>(yv));
-      } else {
-        yv = to_f32(((const act_t*)y)[(size_t)t * W + c]);
-      }
-      float nv[STREAMS_MAX];
-#pragma unroll
-      for (int r = 0; r < STREAMS_MAX; r++) {
-        if (r < S) {
-          float a = 0.f;
-#pragma unroll
-          for (int s = 0; s < STREAMS_MAX; s++)
-            if (s < S) a = fmaf(s_mix[s * S + r], v[s], a);
-          nv[r] = fmaf(s_out[r], yv, a);
+    for (int s = 0; s < STREAMS_MAX; s++)
+      if (s < S) {
+        if (V == 4) {
+          const float4 q = *(const float4*)(x + (size_t)s * W + c);
+          v[s][0] = q.x, v[s][V > 1 ? 1 : 0] = q.y, v[s][V > 2 ? 2 : 0] = q.z, v[s][V > 3 ? 3 : 0] = q.w;
+        } else {
+          v[s][0] = x[(size_t)s * W + c];
         }
       }
+    if (y != nullptr) {
+      float yv[V];
+      if (y_parts > 0) {      // planes of a product that split K: added in order, rounded as the join would
+        const float* p = (const float*)y + (size_t)t * W + c;
+#pragma unroll
+        for (int e = 0; e < V; e++) {
+          float a = p[e];
+          for (int k = 1; k < y_parts; k++) a += p[k * y_plane + e];
+          yv[e] = to_f32(from_f32<act_t>(a));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; e++) yv[e] = to_f32(((const act_t*)y)[(size_t)t * W + c + e]);
+      }
+      float nv[STREAMS_MAX][V];
 #pragma unroll
       for (int r = 0; r < STREAMS_MAX; r++)
         if (r < S) {
-          v[r] = nv[r];
-          x[(size_t)r * W + c] = nv[r];
+#pragma unroll
+          for (int e = 0; e < V; e++) {
+            float a = 0.f;
+#pragma unroll
+            for (int s = 0; s < STREAMS_MAX; s++)
+              if (s < S) a = fmaf(s_mix[s * S + r], v[s][e], a);
+            nv[r][e] = fmaf(s_out[r], yv[e], a);
+          }
+        }
+#pragma unroll
+      for (int r = 0; r < STREAMS_MAX; r++)
+        if (r < S) {
+#pragma unroll
+          for (int e = 0; e < V; e++) v[r][e] = nv[r][e];
+          if (V == 4) {
+            *(float4*)(x + (size_t)r * W + c) = make_float4(nv[r][0], nv[r][V > 1 ? 1 : 0], nv[r][V > 2 ? 2 : 0], nv[r][V > 3 ? 3 : 0]);
+          } else {
+            x[(size_t)r * W + c] = nv[r][0];
+          }
         }
     }
     if (out != nullptr) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < STREAMS_MAX; s++)
-        if (s < S) u = fmaf(s_in[s], v[s], u);
-      u_row[c] = u;
-      sum += u;
+      for (int e = 0; e < V; e++) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; s++)
+          if (s < S) u = fmaf(s_in[s], v[s][e], u);
+        u_row[c + e] = u;
+        sum += u;
+      }
     }
   }
   if (out == nullptr) return;
   const float mean = block_sum(sum, scratch) / (float)W;
   float dev = 0.f;
-  for (int c = tid; c < W; c += 256) {
+  for (int c = tid; c < W; c += nt) {
     const float d = u_row[c] - mean;
     dev = fmaf(d, d, dev);
   }
   const float var = block_sum(dev, scratch) / (float)W;
   const float inv = 1.0f / sqrtf(var + eps);
   act_t* o = out + (size_t)b * W;
-  for (int c = tid; c < W; c += 256) o[c] = from_f32<act_t>(fmaf((u_row[c] - mean) * inv, norm_w[c], norm_b ? norm_b[c] : 0.f));
+  for (int c = tid; c < W; c += nt) o[c] = from_f32<act_t>(fmaf((u_row[c] - mean) * inv, norm_w[c], norm_b ? norm_b[c] : 0.f));
 }
 
 // ---- the short convolution
-__global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __restrict__ w, const float* __restrict__ state,
+// RENEW: every request of the step brings one token, so the thread of (token, channel) is the
+// only one that touches its column of the state and moves it on itself.
+template <bool RENEW>
+__global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __restrict__ w, float* __restrict__ state,
                                   int slot_words, int offset_words, const int* __restrict__ positions,
                                   const int* __restrict__ req_of_token, const int* __restrict__ q_start,
                                   const int* __restrict__ slot_of_req, act_t* __restrict__ out, int W, int taps) {
@@ -119,7 +147,7 @@ __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __re
   }
   const int r = req_of_token[t];
   const int before = t - q_start[r];      // rows of this step in front of t that belong to the same request
-  const float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words;
+  float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words;
   const float x = to_f32(h[(size_t)t * W + c]);
   float acc = 0.f;
   for (int j = 0; j < taps; j++) {
@@ -130,6 +158,10 @@ __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __re
     acc = fmaf(w[(size_t)c * taps + j], v, acc);
   }
   out[(size_t)t * W + c] = from_f32<act_t>(x + acc);
+  if (RENEW) {
+    for (int a = taps - 2; a > 0; a--) st[(size_t)a * W + c] = st[(size_t)(a - 1) * W + c];
+    if (taps > 1) st[c] = x;
+  }
 }
 
 __global__ void short_conv_state_kernel(const act_t* __restrict__ h, float* __restrict__ state, int slot_words,
@@ -196,15 +228,24 @@ int zk_streams_step(float* xs, int S, const void* y, int y_parts, const float* w
   ZK_REQUIRE((size_t)W * 4 <= 96 * 1024, "zk_streams_step: rows of more than 24576 channels are not supported");
   if (n_rows == 0) return 0;
   const size_t lds = out ? (size_t)W * 4 : 0;
+  const bool vec = W % 4 == 0 && (uintptr_t)xs % 16 == 0;
   if (lds > 48 * 1024) {
     static bool raised = false;
     if (!raised) {
-      hipFuncSetAttribute((const void*)streams_step_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      hipFuncSetAttribute((const void*)streams_step_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+      hipFuncSetAttribute((const void*)streams_step_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
       raised = true;
     }
   }
-  streams_step_kernel<<<n_rows, 256, lds, (hipStream_t)stream>>>(xs, S, y, y_parts, (size_t)T * W, w_mix, w_out, w_in,
-                                                                 norm_w, norm_b, eps, rows, (act_t*)out, W);
+  // in the 32-bit library the block is always 256 wide: the order of a row's sums must not follow
+  // from how many rows a step brings
+  const int threads = (ZSE_ACT_BF16 && n_rows <= 64) ? 1024 : 256;
+  if (vec)
+    streams_step_kernel<4><<<n_rows, threads, lds, (hipStream_t)stream>>>(xs, S, y, y_parts, (size_t)T * W, w_mix, w_out, w_in,
+                                                                         norm_w, norm_b, eps, rows, (act_t*)out, W);
+  else
+    streams_step_kernel<1><<<n_rows, threads, lds, (hipStream_t)stream>>>(xs, S, y, y_parts, (size_t)T * W, w_mix, w_out, w_in,
+                                                                         norm_w, norm_b, eps, rows, (act_t*)out, W);
   return zk_launch_status("zk_streams_step");
 }
 
@@ -219,9 +260,25 @@ int zk_short_conv(const void* h, const float* w, const float* state, int slot_wo
   if (T == 0) return 0;
   ZK_REQUIRE(T <= 65535, "zk_short_conv: more than 65535 rows");
   dim3 grid((W + 255) / 256, T);
-  short_conv_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, state, slot_words, offset_words, positions,
-                                                           req_of_token, q_start, slot_of_req, (act_t*)out, W, taps);
+  short_conv_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, (float*)state, slot_words, offset_words,
+                                                                  positions, req_of_token, q_start, slot_of_req,
+                                                                  (act_t*)out, W, taps);
   return zk_launch_status("zk_short_conv");
+}
+
+// The convolution and the renewal of the state in one launch, for steps in which every request
+// brings exactly one token (T rows, T requests).
+int zk_short_conv_token(const void* h, const float* w, float* state, int slot_words, int offset_words,
+                        const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                        void* out, int T, int W, int taps, void* stream) {
+  ZK_REQUIRE(T >= 0 && T <= 65535 && W > 0 && taps >= 1, "zk_short_conv_token: bad sizes");
+  ZK_REQUIRE(taps == 1 || (state != nullptr && slot_words >= offset_words + (taps - 1) * W),
+             "zk_short_conv_token: the state does not fit its slot");
+  if (T == 0) return 0;
+  dim3 grid((W + 255) / 256, T);
+  short_conv_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, state, slot_words, offset_words, positions,
+                                                                 req_of_token, q_start, slot_of_req, (act_t*)out, W, taps);
+  return zk_launch_status("zk_short_conv_token");
 }
 
 int zk_short_conv_state(const void* h, float* state, int slot_words, int offset_words, const int* q_start,
@@ -251,5 +308,6 @@ int zk_rotate_heads(void* x, const int* positions, const float* freq, int T, int
 ZK_ENTER(zk_replicate)
 ZK_ENTER(zk_streams_step)
 ZK_ENTER(zk_short_conv)
+ZK_ENTER(zk_short_conv_token)
 ZK_ENTER(zk_short_conv_state)
 ZK_ENTER(zk_rotate_heads)

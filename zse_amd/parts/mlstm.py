@@ -83,8 +83,10 @@ class MatrixMemory(Part):
             k.zk_mlstm_finish(o_raw.ptr, qkvz.ptr, ld, self.gain.ptr, nm.ptr, ctx.state.ptr, words, at, ctx.req_of_token,
                               ctx.q_start, ctx.slot_of_req, out.ptr, T, H, D, E, float(s.eps), ctx.stream)
         else:
-            k.zk_mlstm(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, self.gain.ptr, ctx.state.ptr, words, at,
-                       ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, D, E, float(s.gate_cap), float(s.eps), ctx.stream)
+            # steps of single tokens renew the state where it lies; same bits as the staged kernel
+            run = k.zk_mlstm_token if ctx.max_q_len == 1 else k.zk_mlstm
+            run(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, self.gain.ptr, ctx.state.ptr, words, at,
+                ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, D, E, float(s.gate_cap), float(s.eps), ctx.stream)
         return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 

@@ -38,6 +38,11 @@ class ShortConv(Part):
         out = ctx.alloc((T, s.size))
         state = ctx.state.ptr if ctx.state is not None else None
         words = ctx.state.shape[1] if ctx.state is not None else 0
+        if ctx.max_q_len == 1 and T == ctx.R:
+            # every request brings one token: one launch computes and moves the state on
+            k.zk_short_conv_token(x.ptr, self.weight.ptr, state, words, state_offset // 4, ctx.positions,
+                                  ctx.req_of_token, ctx.q_start, ctx.slot_of_req, out.ptr, T, s.size, s.taps, ctx.stream)
+            return out
         k.zk_short_conv(x.ptr, self.weight.ptr, state, words, state_offset // 4, ctx.positions, ctx.req_of_token,
                         ctx.q_start, ctx.slot_of_req, out.ptr, T, s.size, s.taps, ctx.stream)
         k.zk_short_conv_state(x.ptr, state, words, state_offset // 4, ctx.q_start, ctx.slot_of_req, ctx.R, s.size,

@@ -167,10 +167,12 @@ KERNEL_SIGNATURES = {
     "zk_replicate": [_VP, _VP, _I, _I, _I, _VP],
     "zk_streams_step": [_VP, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _F, _VP, _VP, _I, _I, _I, _VP],
     "zk_short_conv": [_VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _VP],
+    "zk_short_conv_token": [_VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _VP],
     "zk_short_conv_state": [_VP, _VP, _I, _I, _VP, _VP, _I, _I, _I, _VP],
     "zk_rotate_heads": [_VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
     "zk_head_prep": [_VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
     "zk_mlstm": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
+    "zk_mlstm_token": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
     "zk_mlstm_chunked": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
     "zk_mlstm_finish": [_VP, _VP, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
 }
