@@ -136,11 +136,13 @@ def test_matrix_memory_cut_into_steps(dev, H, D, E):
         assert not rt.download(state)[0].any()
 
 
+@pytest.mark.parametrize("side_by_side", [False, True])
 @pytest.mark.parametrize("H,D,E", [(1, 8, 8), (3, 12, 20), (2, 64, 128), (1, 128, 48), (1, 256, 40)])
-def test_matrix_memory_in_chunks(dev, H, D, E):
+def test_matrix_memory_in_chunks(dev, H, D, E, side_by_side):
     """The chunked form of the recurrence with its finishing kernel: two requests side by side,
     portions of 1 to 150 tokens (chunks of 16, 32 and 64; full, partial and single-token ones),
-    continuing from the state the portion before left."""
+    continuing from the state the portion before left.  ``side_by_side``: the three launches that
+    run a step's chunks at once, instead of the kernel that walks them."""
     rt, k = dev
     rng = np.random.default_rng(D + E)
     W = 16
@@ -172,10 +174,16 @@ def test_matrix_memory_in_chunks(dev, H, D, E):
         q_start, req = i32(rt, [0, n0, T]), i32(rt, [0] * n0 + [1] * n1)
         d_slots = i32(rt, slots)
         o_raw, nm, d_o = rt.zeros((T, H * E), "float32"), rt.zeros((2, H * (D + 1)), "float32"), rt.empty((T, H * E), "float32")
-        k.zk_mlstm_chunked(d_rows.ptr, rows.shape[1], d_g.ptr, bi.ptr, bf.ptr, state.ptr, words, 4, q_start.ptr, d_slots.ptr,
-                           o_raw.ptr, nm.ptr, 2, H, D, E, 5.0, max(n0, n1), rt.stream)
-        k.zk_mlstm_finish(o_raw.ptr, d_rows.ptr, rows.shape[1], g.ptr, nm.ptr, state.ptr, words, 4, req.ptr, q_start.ptr,
-                          d_slots.ptr, d_o.ptr, T, H, D, E, 1e-6, rt.stream)
+        if side_by_side:
+            floats = k.zk_mlstm_scan_floats(T, 2, H, D, E, max(n0, n1))
+            work = rt.zeros((floats,), "float32")
+            k.zk_mlstm_scan(d_rows.ptr, rows.shape[1], d_g.ptr, bi.ptr, bf.ptr, state.ptr, words, 4, q_start.ptr, d_slots.ptr,
+                            o_raw.ptr, work.ptr, floats, T, 2, H, D, E, 5.0, max(n0, n1), rt.stream)
+        else:
+            k.zk_mlstm_chunked(d_rows.ptr, rows.shape[1], d_g.ptr, bi.ptr, bf.ptr, state.ptr, words, 4, q_start.ptr, d_slots.ptr,
+                               o_raw.ptr, nm.ptr, 2, H, D, E, 5.0, max(n0, n1), rt.stream)
+        k.zk_mlstm_finish(o_raw.ptr, d_rows.ptr, rows.shape[1], g.ptr, None if side_by_side else nm.ptr, state.ptr, words, 4,
+                          req.ptr, q_start.ptr, d_slots.ptr, d_o.ptr, T, H, D, E, 1e-6, rt.stream)
         o = rt.download(d_o)
         got[0].append(o[:n0])
         got[1].append(o[n0:])

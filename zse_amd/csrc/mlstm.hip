@@ -381,11 +381,315 @@ __global__ __launch_bounds__(64) void mlstm_finish_kernel(
     const float y = o[e] * inv * norm_w[(size_t)hd * E + e] * (1.0f / (1.0f + expf(-to_f32(z[e]))));
     out[((size_t)t * H + hd) * E + e] = from_f32<act_t>(y);
   }
+  if (nm_new == nullptr) return;
   const int r = req_of_token[t];
   if (t == q_start[r + 1] - 1) {
     float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * ((size_t)D * E + D + 1) + (size_t)D * E;
     const float* nm = nm_new + ((size_t)r * H + hd) * (D + 1);
     for (int d = lane; d <= D; d += 64) st[d] = nm[d];
+  }
+}
+
+// ---- the chunks of long portions side by side, in three launches.
+//
+// The chunk kernel above walks a request's chunks one after the other, since each starts from the
+// state the one before left: a head keeps at most a few blocks busy however long the portion.
+// What a chunk adds to the state does not depend on that state, though:
+//
+//   local  (every chunk at once):   A = max_s a_s,  U = sum_s exp(a_s - A) k_s v_s^T,  u likewise,  F = F_L
+//   scan   (chunk after chunk, one multiply-add per element of the state):
+//          M = max(m0, A),  S0' = exp(m0 - M) S0 + exp(A - M) U,  m0' = F + M;   S0, n0, m0 of every chunk are kept
+//   output (every chunk at once):   the read-out of the chunk kernel from the kept S0, n0, m0
+//
+// Chunks are numbered through the step's requests (request r has ceil(n_r / L) of them); a block
+// finds its request by walking q_start.  U is stored where the scan then leaves S0 of that chunk.
+__device__ __forceinline__ bool mlstm_find_chunk(const int* __restrict__ q_start, int R, int L, int x, int& r, int& c0,
+                                                 int& Lc) {
+  int acc = 0;
+  for (r = 0; r < R; r++) {
+    const int t0 = q_start[r], n = q_start[r + 1] - t0;
+    const int nc = (n + L - 1) / L;
+    if (x < acc + nc) {
+      c0 = t0 + (x - acc) * L;
+      Lc = min(L, t0 + n - c0);
+      return true;
+    }
+    acc += nc;
+  }
+  return false;
+}
+
+// Loads a chunk's k (and q) rows and its slice of v into the local memory, zero beyond Lc.
+template <int L, bool WITH_Q>
+__device__ __forceinline__ void mlstm_load_chunk(const act_t* __restrict__ qkvz, int ld, int c0, int Lc, int hd, int e0, int H,
+                                                 int D, int E, float q_scale, float* Qs, float* Ks, float* Vs) {
+  const int tid = threadIdx.x, DP = D + 1;
+  const bool vec8 = D % 8 == 0 && ld % 8 == 0 && (uintptr_t)qkvz % 16 == 0;
+  if (vec8) {
+    const int D8 = D / 8;
+    for (int i = tid; i < L * D8; i += MLSTM_THREADS) {
+      const int j = i / D8, d = (i % D8) * 8;
+      float q[8] = {}, k[8] = {};
+      if (j < Lc) {
+        const act_t* row = qkvz + (size_t)(c0 + j) * ld;
+        if (WITH_Q) load8(row + (size_t)hd * D + d, q);
+        load8(row + (size_t)(H + hd) * D + d, k);
+      }
+#pragma unroll
+      for (int x = 0; x < 8; x++) {
+        if (WITH_Q) Qs[j * DP + d + x] = q[x] * q_scale;
+        Ks[j * DP + d + x] = k[x];
+      }
+    }
+  } else {
+    for (int i = tid; i < L * D; i += MLSTM_THREADS) {
+      const int j = i / D, d = i % D;
+      float q = 0.f, k = 0.f;
+      if (j < Lc) {
+        const act_t* row = qkvz + (size_t)(c0 + j) * ld;
+        if (WITH_Q) q = to_f32(row[(size_t)hd * D + d]) * q_scale;
+        k = to_f32(row[(size_t)(H + hd) * D + d]);
+      }
+      if (WITH_Q) Qs[j * DP + d] = q;
+      Ks[j * DP + d] = k;
+    }
+  }
+  for (int i = tid; i < L * MLSTM_EC; i += MLSTM_THREADS) {
+    const int j = i / MLSTM_EC, e = e0 + i % MLSTM_EC;
+    Vs[i] = (j < Lc && e < E) ? to_f32(qkvz[(size_t)(c0 + j) * ld + (size_t)2 * H * D + (size_t)hd * E + e]) : 0.f;
+  }
+}
+
+template <int L>
+__global__ __launch_bounds__(MLSTM_THREADS) void mlstm_local_kernel(
+    const act_t* __restrict__ qkvz, int ld, const float* __restrict__ gates, const float* __restrict__ bias_i,
+    const float* __restrict__ bias_f, const int* __restrict__ q_start, float* __restrict__ Uw, float* __restrict__ uw,
+    float* __restrict__ af, int R, int H, int D, int E, float cap) {
+  constexpr int EC = MLSTM_EC;
+  extern __shared__ float lds[];
+  const int x = blockIdx.x, hd = blockIdx.y, e0 = blockIdx.z * EC, tid = threadIdx.x;
+  int r, c0, Lc;
+  if (!mlstm_find_chunk(q_start, R, L, x, r, c0, Lc)) return;
+  const int DP = D + 1;
+  float* Ks = lds;                       // [L][DP]
+  float* Vs = Ks + (size_t)L * DP;       // [L][EC]
+  float* ga = Vs + (size_t)L * EC;
+  float* gF = ga + L;
+  float* gw = gF + L;
+  mlstm_load_chunk<L, false>(qkvz, ld, c0, Lc, hd, e0, H, D, E, 0.f, nullptr, Ks, Vs);
+  if (tid < ZSE_WAVE) {
+    const int j = tid;
+    float F = 0.f, gi = 0.f;
+    if (j < Lc) {
+      const size_t t = c0 + j;
+      gi = cap * tanhf((gates[t * 2 * H + hd] + bias_i[hd]) / cap);
+      F = log_sigmoid(cap * tanhf((gates[t * 2 * H + H + hd] + bias_f[hd]) / cap));
+    }
+#pragma unroll
+    for (int o = 1; o < ZSE_WAVE; o <<= 1) {
+      const float up = __shfl_up(F, o, ZSE_WAVE);
+      if (j >= o) F += up;
+    }
+    const float a = j < Lc ? gi - F : -INFINITY;
+    const float A = wave_max(a);
+    if (j < L) gw[j] = j < Lc ? expf(a - A) : 0.f;
+    if (j == Lc - 1 && blockIdx.z == 0) {
+      af[((size_t)x * H + hd) * 2] = A;
+      af[((size_t)x * H + hd) * 2 + 1] = F;
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < L * EC; i += MLSTM_THREADS) Vs[i] *= gw[i / EC];
+  if (blockIdx.z == 0)
+    for (int d = tid; d < D; d += MLSTM_THREADS) {
+      float acc = 0.f;
+      for (int s2 = 0; s2 < Lc; s2++) acc = fmaf(gw[s2], Ks[s2 * DP + d], acc);
+      uw[((size_t)x * H + hd) * D + d] = acc;
+    }
+  __syncthreads();
+  float* U = Uw + ((size_t)x * H + hd) * D * E;
+  const int ec = (tid % 16) * 2, dg = (tid / 16) * 4;
+  for (int db = 0; db < D; db += 64) {
+    float acc[4][2] = {};
+    const int d = db + dg;
+    for (int s2 = 0; s2 < Lc; s2++) {
+      const float v0 = Vs[s2 * EC + ec], v1 = Vs[s2 * EC + ec + 1];
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        const float k = d + a < D ? Ks[s2 * DP + d + a] : 0.f;
+        acc[a][0] = fmaf(k, v0, acc[a][0]);
+        acc[a][1] = fmaf(k, v1, acc[a][1]);
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+      if (d + a < D) {
+        if (e0 + ec < E) U[(size_t)(d + a) * E + e0 + ec] = acc[a][0];
+        if (e0 + ec + 1 < E) U[(size_t)(d + a) * E + e0 + ec + 1] = acc[a][1];
+      }
+  }
+}
+
+// One thread per element of a head's state (S, then n, then one more thread that keeps m).
+__global__ __launch_bounds__(MLSTM_THREADS) void mlstm_scan_kernel(
+    float* __restrict__ state, int slot_words, int offset_words, const int* __restrict__ q_start,
+    const int* __restrict__ slot_of_req, float* __restrict__ Uw, float* __restrict__ uw, const float* __restrict__ af,
+    float* __restrict__ mprev, int L, int H, int D, int E) {
+  const int r = blockIdx.x, hd = blockIdx.y;
+  const int idx = blockIdx.z * MLSTM_THREADS + threadIdx.x;
+  const int DE = D * E;
+  if (idx > DE + D) return;
+  const int t0 = q_start[r], n = q_start[r + 1] - t0;
+  if (n <= 0) return;
+  int first = 0;
+  for (int r2 = 0; r2 < r; r2++) first += (q_start[r2 + 1] - q_start[r2] + L - 1) / L;
+  const int nc = (n + L - 1) / L;
+  float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)hd * ((size_t)DE + D + 1);
+  float m = st[DE + D];
+  float val = idx < DE + D ? st[idx] : 0.f;
+  for (int ci = 0; ci < nc; ci++) {
+    const size_t at = (size_t)(first + ci) * H + hd;
+    const float A = af[at * 2], F = af[at * 2 + 1];
+    const float M = fmaxf(m, A);
+    if (idx < DE + D) {
+      float* p = idx < DE ? Uw + at * DE + idx : uw + at * D + (idx - DE);
+      const float U = *p;
+      *p = val;                                   // the state this chunk starts from
+      val = fmaf(expf(m - M), val, expf(A - M) * U);
+    } else {
+      mprev[at] = m;
+    }
+    m = F + M;
+  }
+  st[idx] = idx < DE + D ? val : m;
+}
+
+template <int L>
+__global__ __launch_bounds__(MLSTM_THREADS) void mlstm_output_kernel(
+    const act_t* __restrict__ qkvz, int ld, const float* __restrict__ gates, const float* __restrict__ bias_i,
+    const float* __restrict__ bias_f, const int* __restrict__ q_start, const float* __restrict__ Sw,
+    const float* __restrict__ nw, const float* __restrict__ mprev, float* __restrict__ o_raw, int R, int H, int D, int E,
+    float cap, float q_scale) {
+  constexpr int EC = MLSTM_EC;
+  constexpr int TP = L / 16;
+  extern __shared__ float lds[];
+  const int x = blockIdx.x, hd = blockIdx.y, e0 = blockIdx.z * EC, tid = threadIdx.x;
+  int r, c0, Lc;
+  if (!mlstm_find_chunk(q_start, R, L, x, r, c0, Lc)) return;
+  const int DP = D + 1, LP = L + 1;
+  float* Ss = lds;
+  float* ns = Ss + (size_t)D * EC;
+  float* Qs = ns + D;
+  float* Ks = Qs + (size_t)L * DP;
+  float* Vs = Ks + (size_t)L * DP;
+  float* Ps = Vs + (size_t)L * EC;
+  float* ga = Ps + (size_t)L * LP;
+  float* gM = ga + L;
+  float* gF = gM + L;
+  float* gden = gF + L;
+  const size_t at = (size_t)x * H + hd;
+  const float* S0 = Sw + at * D * E;
+  for (int i = tid; i < D * EC; i += MLSTM_THREADS) {
+    const int d = i / EC, e = e0 + i % EC;
+    Ss[i] = e < E ? S0[(size_t)d * E + e] : 0.f;
+  }
+  for (int d = tid; d < D; d += MLSTM_THREADS) ns[d] = nw[at * D + d];
+  const float m_prev = mprev[at];
+  mlstm_load_chunk<L, true>(qkvz, ld, c0, Lc, hd, e0, H, D, E, q_scale, Qs, Ks, Vs);
+  if (tid < ZSE_WAVE) {
+    const int j = tid;
+    float F = 0.f, gi = 0.f;
+    if (j < Lc) {
+      const size_t t = c0 + j;
+      gi = cap * tanhf((gates[t * 2 * H + hd] + bias_i[hd]) / cap);
+      F = log_sigmoid(cap * tanhf((gates[t * 2 * H + H + hd] + bias_f[hd]) / cap));
+    }
+#pragma unroll
+    for (int o = 1; o < ZSE_WAVE; o <<= 1) {
+      const float up = __shfl_up(F, o, ZSE_WAVE);
+      if (j >= o) F += up;
+    }
+    const float a = j < Lc ? gi - F : -INFINITY;
+    float M = a;
+#pragma unroll
+    for (int o = 1; o < ZSE_WAVE; o <<= 1) {
+      const float up = __shfl_up(M, o, ZSE_WAVE);
+      if (j >= o) M = fmaxf(M, up);
+    }
+    if (j < L) {
+      ga[j] = a;
+      gM[j] = fmaxf(M, m_prev);
+      gF[j] = F;
+    }
+  }
+  __syncthreads();
+  {
+    const int pj = tid / 16, ps = tid % 16;
+    float acc[TP][TP] = {};
+    for (int d = 0; d < D; d++) {
+      float q[TP], k[TP];
+#pragma unroll
+      for (int y = 0; y < TP; y++) {
+        q[y] = Qs[(pj + 16 * y) * DP + d];
+        k[y] = Ks[(ps + 16 * y) * DP + d];
+      }
+#pragma unroll
+      for (int a = 0; a < TP; a++)
+#pragma unroll
+        for (int b = 0; b < TP; b++) acc[a][b] = fmaf(q[a], k[b], acc[a][b]);
+    }
+#pragma unroll
+    for (int a = 0; a < TP; a++)
+#pragma unroll
+      for (int b = 0; b < TP; b++) {
+        const int j = pj + 16 * a, s2 = ps + 16 * b;
+        Ps[j * LP + s2] = (s2 <= j && j < Lc) ? acc[a][b] * expf(ga[s2] - gM[j]) : 0.f;
+      }
+  }
+  __syncthreads();
+  if (tid < L) {
+    const int j = tid;
+    float nq = 0.f;
+    for (int d = 0; d < D; d++) nq = fmaf(ns[d], Qs[j * DP + d], nq);
+    nq *= expf(m_prev - gM[j]);
+    for (int s2 = 0; s2 <= j; s2++) nq += Ps[j * LP + s2];
+    gden[j] = fmaxf(fabsf(nq), expf(-(gF[j] + gM[j]))) + 1e-6f;
+  }
+  const int ec = (tid % 16) * 2, rg = tid / 16;
+  float acc[TP][2] = {};
+  for (int d = 0; d < D; d++) {
+    const float s0 = Ss[d * EC + ec], s1 = Ss[d * EC + ec + 1];
+#pragma unroll
+    for (int a = 0; a < TP; a++) {
+      const float q = Qs[(rg + 16 * a) * DP + d];
+      acc[a][0] = fmaf(q, s0, acc[a][0]);
+      acc[a][1] = fmaf(q, s1, acc[a][1]);
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < TP; a++) {
+    const float g = expf(m_prev - gM[rg + 16 * a]);
+    acc[a][0] *= g;
+    acc[a][1] *= g;
+  }
+  for (int s2 = 0; s2 < Lc; s2++) {
+    const float v0 = Vs[s2 * EC + ec], v1 = Vs[s2 * EC + ec + 1];
+#pragma unroll
+    for (int a = 0; a < TP; a++) {
+      const float p = Ps[(rg + 16 * a) * LP + s2];
+      acc[a][0] = fmaf(p, v0, acc[a][0]);
+      acc[a][1] = fmaf(p, v1, acc[a][1]);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < TP; a++) {
+    const int j = rg + 16 * a;
+    if (j < Lc) {
+      float* o = o_raw + ((size_t)(c0 + j) * H + hd) * E;
+      if (e0 + ec < E) o[e0 + ec] = acc[a][0] / gden[j];
+      if (e0 + ec + 1 < E) o[e0 + ec + 1] = acc[a][1] / gden[j];
+    }
   }
 }
 
@@ -487,6 +791,79 @@ int zk_mlstm_chunked(const void* qkvz, int ld, const float* gates, const float* 
 #undef ZK_CHUNK_
 }
 
+}  // extern "C"
+
+static int mlstm_scan_len(int max_q_len, int D) {
+  int L = max_q_len <= 16 ? 16 : max_q_len <= 32 ? 32 : 64;
+  while (L > 16 && mlstm_chunk_lds(L, D) > 150 * 1024) L /= 2;
+  return L;
+}
+
+// Floats of scratch that zk_mlstm_scan needs for a step of T tokens in R requests.
+extern "C" size_t zk_mlstm_scan_floats(int T, int R, int H, int D, int E, int max_q_len) {
+  const int L = mlstm_scan_len(max_q_len, D);
+  const size_t chunks = (size_t)(T + L - 1) / L + R;
+  return chunks * H * ((size_t)D * E + D + 3);
+}
+
+template <int L>
+static int mlstm_scan_launch(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f,
+                             float* state, int slot_words, int offset_words, const int* q_start, const int* slot_of_req,
+                             float* o_raw, float* work, int chunks, int R, int H, int D, int E, float cap, hipStream_t s) {
+  float* Uw = work;
+  float* uw = Uw + (size_t)chunks * H * D * E;
+  float* af = uw + (size_t)chunks * H * D;
+  float* mprev = af + (size_t)chunks * H * 2;
+  const int zs = (E + MLSTM_EC - 1) / MLSTM_EC;
+  const size_t lds_local = ((size_t)L * (D + 1) + (size_t)L * MLSTM_EC + 3 * L + 8) * 4;
+  const size_t lds_out = mlstm_chunk_lds(L, D);
+  static size_t raised_local = 0, raised_out = 0;
+  if (lds_local > 48 * 1024 && lds_local > raised_local) {
+    hipFuncSetAttribute((const void*)mlstm_local_kernel<L>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_local);
+    raised_local = lds_local;
+  }
+  if (lds_out > 48 * 1024 && lds_out > raised_out) {
+    hipFuncSetAttribute((const void*)mlstm_output_kernel<L>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_out);
+    raised_out = lds_out;
+  }
+  mlstm_local_kernel<L><<<dim3(chunks, H, zs), MLSTM_THREADS, lds_local, s>>>((const act_t*)qkvz, ld, gates, bias_i, bias_f,
+                                                                              q_start, Uw, uw, af, R, H, D, E, cap);
+  if (int rc = zk_launch_status("zk_mlstm_scan (local)")) return rc;
+  mlstm_scan_kernel<<<dim3(R, H, (D * E + D + 1 + MLSTM_THREADS - 1) / MLSTM_THREADS), MLSTM_THREADS, 0, s>>>(
+      state, slot_words, offset_words, q_start, slot_of_req, Uw, uw, af, mprev, L, H, D, E);
+  if (int rc = zk_launch_status("zk_mlstm_scan (scan)")) return rc;
+  mlstm_output_kernel<L><<<dim3(chunks, H, zs), MLSTM_THREADS, lds_out, s>>>((const act_t*)qkvz, ld, gates, bias_i, bias_f,
+                                                                             q_start, Uw, uw, mprev, o_raw, R, H, D, E, cap,
+                                                                             1.0f / sqrtf((float)D));
+  return zk_launch_status("zk_mlstm_scan (output)");
+}
+
+extern "C" {
+
+// zk_mlstm_chunked's work with the chunks of a step side by side (three launches); for steps
+// whose portions are several chunks long.  work: zk_mlstm_scan_floats(...) floats of scratch.
+// zk_mlstm_finish (with nm_new null: the scan stores n and m itself) must follow.
+int zk_mlstm_scan(const void* qkvz, int ld, const float* gates, const float* bias_i, const float* bias_f, float* state,
+                  int slot_words, int offset_words, const int* q_start, const int* slot_of_req, float* o_raw, float* work,
+                  size_t work_floats, int T, int R, int H, int D, int E, float cap, int max_q_len, void* stream) {
+  ZK_REQUIRE(T >= 0 && R >= 0 && R <= 65535 && H > 0 && H <= 65535 && D > 0 && E > 0, "zk_mlstm_scan: bad sizes");
+  ZK_REQUIRE(D <= 256 && E <= 2048, "zk_mlstm_scan: heads of more than 256 key channels are not supported");
+  ZK_REQUIRE(ld >= 2 * H * (D + E), "zk_mlstm_scan: rows too short");
+  ZK_REQUIRE(cap > 0.f, "zk_mlstm_scan: the gates' cap must be positive");
+  ZK_REQUIRE((size_t)slot_words * 4 >= (size_t)offset_words * 4 + zk_mlstm_state_bytes(H, D, E),
+             "zk_mlstm_scan: the state does not fit its slot");
+  ZK_REQUIRE(work != nullptr && work_floats >= zk_mlstm_scan_floats(T, R, H, D, E, max_q_len), "zk_mlstm_scan: too little scratch");
+  if (R == 0 || T == 0) return 0;
+  const int L = mlstm_scan_len(max_q_len, D);
+  const int chunks = (T + L - 1) / L + R;
+  hipStream_t s = (hipStream_t)stream;
+#define ZK_SCAN_(L_) \
+  mlstm_scan_launch<L_>(qkvz, ld, gates, bias_i, bias_f, state, slot_words, offset_words, q_start, slot_of_req, o_raw, work, \
+                        chunks, R, H, D, E, cap, s)
+  return L == 64 ? ZK_SCAN_(64) : L == 32 ? ZK_SCAN_(32) : ZK_SCAN_(16);
+#undef ZK_SCAN_
+}
+
 int zk_mlstm_finish(const float* o_raw, const void* qkvz, int ld, const float* norm_w, const float* nm_new,
                     float* state, int slot_words, int offset_words, const int* req_of_token, const int* q_start,
                     const int* slot_of_req, void* out, int T, int H, int D, int E, float eps, void* stream) {
@@ -504,4 +881,5 @@ int zk_mlstm_finish(const float* o_raw, const void* qkvz, int ld, const float* n
 ZK_ENTER(zk_mlstm)
 ZK_ENTER(zk_mlstm_token)
 ZK_ENTER(zk_mlstm_chunked)
+ZK_ENTER(zk_mlstm_scan)
 ZK_ENTER(zk_mlstm_finish)

@@ -12,7 +12,8 @@ at zero and is carried as floats in the request's state slot:
 q, k, v and z are one product; the two gates are a second, small one whose results stay float.
 Steps of single tokens run the recurrence as written, one block per (request, head); steps with
 portions of prompts run it over chunks of up to 64 tokens, where it becomes four small matrix
-products per chunk, with a head's value channels spread over several blocks.
+products per chunk, with a head's value channels spread over several blocks; portions of several
+chunks run all their chunks at once around a short scan that carries the state from chunk to chunk.
 """
 from __future__ import annotations
 
@@ -25,6 +26,7 @@ from .ops import linear
 
 class MatrixMemory(Part):
     graph_safe = True      # rows, requests and slots are read by the kernel from device memory
+    SCAN_FROM = 64         # portions longer than this (more than one chunk) run their chunks side by side
 
     def __init__(self, spec):
         s = self.spec = spec
@@ -76,11 +78,22 @@ class MatrixMemory(Part):
             # heads' norm and gate.  (In 32-bit every step runs token by token, so that a request's
             # values are the same bits however its tokens are cut into steps.)
             o_raw = ctx.alloc((T, H * E), F32)
-            nm = ctx.alloc((ctx.R, H * (D + 1)), F32)
-            k.zk_mlstm_chunked(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, ctx.state.ptr, words, at,
-                               ctx.q_start, ctx.slot_of_req, o_raw.ptr, nm.ptr, ctx.R, H, D, E, float(s.gate_cap),
-                               int(ctx.max_q_len), ctx.stream)
-            k.zk_mlstm_finish(o_raw.ptr, qkvz.ptr, ld, self.gain.ptr, nm.ptr, ctx.state.ptr, words, at, ctx.req_of_token,
+            if ctx.max_q_len > self.SCAN_FROM:
+                # portions of several chunks: every chunk's own part at once, a short scan over the
+                # chunks, every chunk's read-out at once
+                floats = int(k.zk_mlstm_scan_floats(T, ctx.R, H, D, E, int(ctx.max_q_len)))
+                work = ctx.alloc((floats,), F32)
+                k.zk_mlstm_scan(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, ctx.state.ptr, words, at,
+                                ctx.q_start, ctx.slot_of_req, o_raw.ptr, work.ptr, floats, T, ctx.R, H, D, E,
+                                float(s.gate_cap), int(ctx.max_q_len), ctx.stream)
+                nm_ptr = None
+            else:
+                nm = ctx.alloc((ctx.R, H * (D + 1)), F32)
+                k.zk_mlstm_chunked(qkvz.ptr, ld, gates.ptr, self.bias_i.ptr, self.bias_f.ptr, ctx.state.ptr, words, at,
+                                   ctx.q_start, ctx.slot_of_req, o_raw.ptr, nm.ptr, ctx.R, H, D, E, float(s.gate_cap),
+                                   int(ctx.max_q_len), ctx.stream)
+                nm_ptr = nm.ptr
+            k.zk_mlstm_finish(o_raw.ptr, qkvz.ptr, ld, self.gain.ptr, nm_ptr, ctx.state.ptr, words, at, ctx.req_of_token,
                               ctx.q_start, ctx.slot_of_req, out.ptr, T, H, D, E, float(s.eps), ctx.stream)
         else:
             # steps of single tokens renew the state where it lies; same bits as the staged kernel

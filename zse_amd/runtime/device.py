@@ -174,6 +174,7 @@ KERNEL_SIGNATURES = {
     "zk_mlstm": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
     "zk_mlstm_token": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _F, _F, _VP],
     "zk_mlstm_chunked": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
+    "zk_mlstm_scan": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_mlstm_finish": [_VP, _VP, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
 }
 # present only in the bf16 library
@@ -264,6 +265,8 @@ class KernelLibrary:
             setattr(self, name, fn)
         self._dll.zk_mlstm_state_bytes.restype, self._dll.zk_mlstm_state_bytes.argtypes = C.c_size_t, [_I, _I, _I]
         self.zk_mlstm_state_bytes = self._dll.zk_mlstm_state_bytes
+        self._dll.zk_mlstm_scan_floats.restype, self._dll.zk_mlstm_scan_floats.argtypes = C.c_size_t, [_I] * 6
+        self.zk_mlstm_scan_floats = self._dll.zk_mlstm_scan_floats
         if dtype == BF16:
             self._dll.zk_attention_bf16_supports.restype = C.c_int
             self._dll.zk_attention_bf16_supports.argtypes = [_I, _I, _I, _I]
