@@ -35,7 +35,7 @@ def i32(rt, a):
     return up(rt, np.asarray(a, np.int32))
 
 
-@pytest.mark.parametrize("S,W", [(1, 24), (3, 40), (8, 300)])
+@pytest.mark.parametrize("S,W", [(1, 24), (2, 30), (3, 40), (8, 300)])
 def test_streams_write_read_and_norm(dev, S, W):
     rt, k = dev
     rng = np.random.default_rng(S)

@@ -79,10 +79,19 @@ __global__ __launch_bounds__(MLSTM_THREADS) void mlstm_kernel(
     if (active) {
       const float bv = b * sv[e];
       float acc = 0.f;
-      for (int d = d0; d < d1; d++) {
-        const float s = fmaf(a, S[(size_t)d * E + e], sk[d] * bv);
-        S[(size_t)d * E + e] = s;
-        acc = fmaf(s, sq[d], acc);
+      // eight elements of S are asked for before the first of them is written back: the loads
+      // of a thread's column are then in flight together (the sums keep their order)
+      for (int d = d0; d < d1; d += 8) {
+        float old[8];
+#pragma unroll
+        for (int x = 0; x < 8; x++) old[x] = d + x < d1 ? S[(size_t)(d + x) * E + e] : 0.f;
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+          if (d + x < d1) {
+            const float s = fmaf(a, old[x], sk[d + x] * bv);
+            S[(size_t)(d + x) * E + e] = s;
+            acc = fmaf(s, sq[d + x], acc);
+          }
       }
       part[sl * E + e] = acc;
     }
