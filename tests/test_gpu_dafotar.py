@@ -266,6 +266,22 @@ def test_greedy_generation_through_the_engine(models):
         assert eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0)) == want
 
 
+def test_the_engine_at_its_default_limits(models):
+    """No limits given: the longest sequence is the architecture's own default, the pools follow from the
+    free memory; a model with windows only, and one that keeps every key."""
+    from zse_amd.engine.engine import Engine
+    from zse_amd.sampling.sampler import SamplingParams
+    for name in ("A", "B"):
+        cfg, seed = CONFIGS[name]
+        folder = models[(name, "float32")][0]
+        w = random_weights(cfg, seed)
+        prompt = tokens_of(cfg["vocab"], 19, 500)
+        with Engine(folder, dtype="float32") as eng:
+            assert eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.0)) == [plain_greedy(cfg, w, prompt, 6)]
+        with Engine(models[(name, "bfloat16")][0], dtype="bfloat16") as eng:
+            assert len(eng.generate([prompt], SamplingParams(max_tokens=6, temperature=0.7, top_k=10, seed=1))[0]) == 6
+
+
 def test_generation_in_bfloat16_does_not_depend_on_the_company(models):
     from zse_amd.engine.engine import Engine
     from zse_amd.sampling.sampler import SamplingParams

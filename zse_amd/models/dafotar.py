@@ -27,7 +27,8 @@ from ..config.plan import (AttentionSpec, EmbeddingSpec, GatedMLPSpec, HeadSpec,
                            StreamsBlockSpec)
 
 NAME = "Dafotar"
-MAX_POSITION = 1 << 17        # the config names no longest sequence; tables and pools are sized by the runner's own limits
+MAX_POSITION = 1 << 16        # the config names no longest sequence: the longest the engine's decode attention takes for any head size;
+#                               tables and pools are sized by the runner's own limits
 
 
 @dataclass(frozen=True)
