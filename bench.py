@@ -463,6 +463,57 @@ def state_bytes_touched(model):
     return total
 
 
+def check_design_slice(cfg, rt, seed, std, gain_std, std_of):
+    """The first three layers of the Dafotar model that is timed, at full width, against the plain
+    implementation under ``tests/plain`` on the same weights made on the host: a prompt of 150 tokens
+    whole (the mLSTM's chunks side by side), another in portions and then token by token beside a
+    third, in 32-bit and in bfloat16.  The head is restricted to the first 4,096 rows of the embedding."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from plain import dafotar_plain as P
+    from zse_amd.engine.loading import random_model
+    from zse_amd.engine.model import Model
+    from zse_amd.engine.runner import StepEntry, StepRunner
+    from zse_amd.config.base import resolve_architecture
+    from zse_amd.weights.random_init import random_tensors
+    Vc = min(4096, cfg["vocab"])
+    small = dict(cfg, layers=cfg["layers"][:3])
+    host_cfg = dict(small, vocab=Vc)
+    arch = resolve_architecture(host_cfg)
+    plan = arch.plan(arch.config_from_dict(host_cfg))
+    w32 = random_tensors(Model(plan).tensor_reqs(), seed, std, gain_std, std_of, plan.optional_prefixes)
+    rng = np.random.default_rng(11)
+    streams = {"a": rng.integers(0, Vc, 150).tolist(), "b": rng.integers(0, Vc, 90).tolist(),
+               "c": rng.integers(0, Vc, 21).tolist()}
+    steps = [[("a", 150)], [("b", 70)], [("b", 2), ("c", 5)], [("b", 5), ("c", 1)]]
+    steps += [[("b", 1), ("c", 3 if i == 0 else 1)] for i in range(13)]
+    out = {}
+    for dtype in ("float32", "bfloat16"):
+        w = w32 if dtype == "float32" else {n: bf16_round(t) for n, t in w32.items()}
+        model = random_model(small, dtype, seed=seed, std=std, gain_std=gain_std, rt=rt, std_of=std_of)
+        runner = StepRunner(model, rt, dtype, page_size=16, cache_tokens=512, max_seqs=4, max_batch_tokens=256,
+                            max_model_len=256, use_graphs=False)
+        fed = {r: 0 for r in streams}
+        rows = {r: [] for r in streams}
+        for st in steps:
+            es = [StepEntry(r, streams[r][fed[r]:fed[r] + n], range(n)) for r, n in st if fed[r] < len(streams[r])]
+            z = runner.step(es)
+            at = 0
+            for e in es:
+                n = len(e.tokens)
+                rows[e.req].append(z[at:at + n, :Vc])
+                at += n
+                fed[e.req] += n
+        assert all(fed[r] == len(t) for r, t in streams.items()), fed
+        worst = 0.0
+        for r, toks in streams.items():
+            want = P.forward(host_cfg, w, toks, np.float64)
+            got = np.concatenate(rows[r]).astype(np.float64)
+            worst = max(worst, float(np.abs(got - want).max() / max(1e-9, np.abs(want).max())))
+        out[dtype] = worst
+        del runner, model
+    return out
+
+
 def run_design(a):
     """Prefill and decode of Dafotar beside Gemma 2 at equal layer sizes; one JSON line."""
     from zse_amd.engine.loading import random_model
@@ -474,15 +525,27 @@ def run_design(a):
     for name in sizes:
         size = DESIGN_SIZES[name]
         rec = {"config": size}
+        std_of = {".hc": 0.3, ".temp": 0.5, "canon": 0.3}
         for which, cfg in (("dafotar", dafotar_config(**size)), ("gemma2", gemma2_like(**size))):
             if a.only_model and which != a.only_model:
                 continue
+            if which == "dafotar" and not a.no_check and not a.only:
+                errs = check_design_slice(cfg, rt, 0, 0.02, 0.1, std_of)
+                rec["check"] = {"fp32_max_rel_err": float(f"{errs['float32']:.3g}"), "bf16_max_rel_err": float(f"{errs['bfloat16']:.3g}"),
+                                "slice_layers": 3, "cuts": "whole, portions, token by token, mixed"}
+                log(f"{name} check against the plain implementation: {rec['check']}")
+                if not (errs["float32"] < 1e-4 and errs["bfloat16"] < 0.05):
+                    raise SystemExit(f"bench.py: {name}: the engine does not agree with the plain implementation: {rec['check']}")
             # the streams' weights near the plain residual sum, so that activations keep their size over the layers
-            model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt,
-                                 std_of={".hc": 0.3, ".temp": 0.5, "canon": 0.3})
+            model = random_model(cfg, "bfloat16", seed=0, std=0.02, gain_std=0.1, rt=rt, std_of=std_of)
             tcfg = dict(cfg, vocab_size=size["vocab"])
+            if not a.no_check and a.only != "prefill":
+                # the ids of the timed path (captured graphs, ids fed on the device, the picking head) against
+                # steps launched call by call whose logits the host reads
+                if not check_decode_path(model, rt, size["vocab"], a.batch, not a.no_graphs):
+                    raise SystemExit(f"bench.py: {name} {which}: the timed decode path does not pick the tokens of eager steps")
             t = Timed(model, rt, tcfg, a.batch, a.context, a.prefill_tokens, not a.no_graphs, page=a.page_size)
-            r = {"weights_gb": round(model.weight_bytes / 1e9, 3)}
+            r = {"weights_gb": round(model.weight_bytes / 1e9, 3), "checked": bool(not a.no_check and a.only != "prefill")}
             if a.only != "decode":
                 pre_s, pf = t.prefill()
                 r["prefill"] = {"value": round(a.prefill_tokens / pre_s, 1), "ms": round(pre_s * 1e3, 3),

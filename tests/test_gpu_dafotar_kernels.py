@@ -60,6 +60,25 @@ def test_streams_write_read_and_norm(dev, S, W):
     assert np.abs(rt.download(d_p) - want).max() < 2e-5
 
 
+def test_streams_write_from_partial_sums(dev):
+    """A product that split K hands over float planes [P, T, W]; the kernel adds them up itself."""
+    rt, k = dev
+    rng = np.random.default_rng(9)
+    T, S, W, Pn = 6, 4, 64, 3
+    xs = rng.normal(size=(T, S, W)).astype(np.float32)
+    planes = rng.normal(size=(Pn, T, W)).astype(np.float32)
+    mix, out, win = (rng.normal(size=s).astype(np.float32) for s in ((S, S), (S,), (S,)))
+    g, b = rng.normal(1, 0.2, W).astype(np.float32), rng.normal(0, 0.2, W).astype(np.float32)
+    d_xs, d_o = up(rt, xs), rt.empty((T, W), "float32")
+    k.zk_streams_step(d_xs.ptr, S, up(rt, planes).ptr, Pn, up(rt, mix).ptr, up(rt, out).ptr, up(rt, win).ptr, up(rt, g).ptr,
+                      up(rt, b).ptr, 1e-5, None, d_o.ptr, T, T, W, rt.stream)
+    y = planes[0] + planes[1] + planes[2]
+    want_xs = P.streams_write(xs, mix, out, y, np.float64)
+    want = P.layer_norm(P.streams_read(want_xs, win, np.float64), g, b, 1e-5, np.float64)
+    assert np.abs(rt.download(d_xs) - want_xs).max() < 1e-5
+    assert np.abs(rt.download(d_o) - want).max() < 2e-5
+
+
 @pytest.mark.parametrize("taps", [2, 4, 7])
 def test_short_convolution_over_steps(dev, taps):
     """Two requests whose rows come in portions of unequal sizes, also of one and two rows, side
