@@ -437,7 +437,7 @@ DESIGN_SIZES = {
 def dafotar_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
     att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
            "mask": {"size": window}, "rot": {"base": 10000.0, "dims": dim // 2}}
-    rec = {"heads": heads, "dim": dim // 2, "vdim": dim, "gate_cap": 15.0}
+    rec = {"heads": heads, "dim": dim // 2, "vdim": dim, "gate_cap": 10.0}
     layers = []
     for g in range(groups):
         layers += [{"type": "attention", "mixer": dict(att), "mlp": {"kind": "dense", "ff": ff}},
