@@ -121,7 +121,7 @@ def test_short_convolution_over_steps(dev, taps):
     assert not st[1].any() and not st[:, :8].any() and not st[:, 8 + (taps - 1) * W:].any()     # nothing outside its place
 
 
-@pytest.mark.parametrize("H,D,E", [(1, 8, 8), (3, 12, 20), (2, 64, 128), (2, 20, 256)])
+@pytest.mark.parametrize("H,D,E", [(1, 8, 8), (3, 12, 20), (2, 64, 128), (2, 20, 256), (1, 200, 256)])
 def test_matrix_memory_cut_into_steps(dev, H, D, E):
     rt, k = dev
     rng = np.random.default_rng(D)

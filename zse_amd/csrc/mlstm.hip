@@ -740,6 +740,8 @@ static int mlstm_run(bool direct, const void* qkvz, int ld, const float* gates, 
   ZK_REQUIRE((size_t)slot_words * 4 >= (size_t)offset_words * 4 + zk_mlstm_state_bytes(H, D, E),
              "zk_mlstm: the state does not fit its slot");
   if (R == 0) return 0;
+  // a head's S that does not fit the local memory stays in the state slot (the same bits, slower)
+  if (!direct && ((size_t)D * E + 3 * D + E + MLSTM_THREADS + 32) * 4 > 150 * 1024) direct = true;
   const size_t lds = ((direct ? 0 : (size_t)D * E) + 3 * D + E + MLSTM_THREADS + 32) * 4;
   ZK_REQUIRE(lds <= 160 * 1024, "zk_mlstm: a head's state does not fit the local memory");
   if (lds > 48 * 1024) {
