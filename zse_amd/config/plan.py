@@ -46,8 +46,11 @@ class ShortConvSpec:
     zeros before a sequence's start; the last ``taps - 1`` rows are a request's state."""
     size: int
     taps: int
-    weight: str                      # [size, taps]
+    weight: Any                      # [size, taps]: a name, or several whose tensors are stacked along the channels
     kind: str = "short_conv"
+    residual: bool = True            # False: the sum alone, without x_t added
+    activation: Optional[str] = None  # "silu": applied to the result
+    channel_counts: Optional[Tuple[int, ...]] = None   # with several weight names: the channels of each
 
 
 @dataclass(frozen=True)
@@ -57,6 +60,11 @@ class RotarySpec:
     rotary_dim: int
     theta: float
     kind: str = "rotary"
+    interleaved: bool = False        # pairs (2i, 2i + 1) instead of (i, i + rotary_dim / 2)
+    # (factor, original, fast, slow): frequencies that turn fewer than ``slow`` times in ``original``
+    # positions are divided by ``factor``, those that turn more than ``fast`` times stay, a linear
+    # ramp over the pair numbers in between; sines and cosines are multiplied by 0.1 ln(factor) + 1
+    scaling: Optional[Tuple[float, float, float, float]] = None
 
 
 @dataclass(frozen=True)
@@ -86,6 +94,46 @@ class AttentionSpec:
     value_rotation: Optional[float] = None   # base: values are cached turned by their position over all their
     #                                          channels (pair m by pos * base^(-2m/value_dim)), outputs turned back
     value_pairs_interleaved: bool = False    # pairs (2m, 2m + 1) instead of (m, m + value_dim / 2)
+    biases: Optional[Dict[str, str]] = None  # roles q, k, v, o -> names of vectors added in the projections
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are made from one cached latent row per token:
+    c = rms_norm(first ``latent_dim`` rows of W_down x) * gain; the last ``rotary_dim`` rows, rotated,
+    are a key part that all heads share.  Head h's key is [W_uk,h c, rotated part], its value
+    W_uv,h c; a query head has ``head_dim`` plain and ``rotary_dim`` rotated channels.
+    ``sinks``: a learned number per head whose exponential joins the softmax's denominator."""
+    hidden_size: int
+    num_heads: int
+    head_dim: int                    # unrotated query/key channels of a head
+    rotary_dim: int                  # rotated ones (the shared key part's size)
+    value_dim: int
+    latent_dim: int
+    scale: float
+    eps: float                       # of the latent's norm
+    position: Any                    # a rotary spec over rotary_dim channels
+    names: Dict[str, str]            # roles q, down, down_norm, up_k, up_v, o, sinks (optional)
+    window: Optional[int] = None
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """A recurrent mixer with a matrix state per head, written by the gated delta rule:
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with q and k unit vectors (q times
+    key_dim^(-1/2)), beta = sigmoid(W_b x), g = exp(-exp(A) softplus(W_a x + dt)); q, k, v pass a
+    short causal convolution and silu first; the read-out is divided by its root mean square per
+    head, times a gain [value_dim] and silu(W_g x)."""
+    hidden_size: int
+    num_heads: int                   # value heads
+    num_kv_heads: int                # query/key heads; value head h reads head h // (num_heads / num_kv_heads)
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    eps: float
+    names: Dict[str, str]            # roles q, k, v, q_conv, k_conv, v_conv, b, a, A_log, dt_bias, norm, gate, o
+    kind: str = "delta_rule"
 
 
 @dataclass(frozen=True)
@@ -108,9 +156,30 @@ class GatedMLPSpec:
     """act(x Wg^T) * (x Wu^T), then Wd^T."""
     hidden_size: int
     intermediate_size: int
-    activation: str                  # "gelu_tanh" | "silu"
+    activation: str                  # "gelu_tanh" | "silu" | "relu" | "clamped_swiglu"
     names: Dict[str, str]            # roles gate, up, down
     kind: str = "gated_mlp"
+    # clamped_swiglu: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1)
+    limit: Optional[float] = None
+
+
+@dataclass(frozen=True)
+class RoutedMLPSpec:
+    """A mixture of ``num_experts`` gated layers of which a token uses ``top_k``: scores
+    sigmoid(W_router x), the largest chosen, the chosen scores themselves as weights (not
+    renormalised).  ``scale_input``: the weight multiplies the expert's input, expert(w x), not its
+    output.  ``shared``: a gated layer that every token passes, added to the sum (or None)."""
+    hidden_size: int
+    intermediate_size: int           # of one expert
+    num_experts: int
+    top_k: int
+    activation: str                  # as GatedMLPSpec's
+    limit: Optional[float]
+    router: str                      # [num_experts, hidden]
+    expert_names: str                # a pattern with {e} and {role}: role is gate, up or down
+    shared: Any = None               # a GatedMLPSpec or None
+    scale_input: bool = True
+    kind: str = "routed_mlp"
 
 
 @dataclass(frozen=True)
@@ -120,6 +189,7 @@ class BlockSpec:
     ``arrangement``:
       "sandwich": h += post_m(mixer(pre_m(h))); h += post_f(ffn(pre_f(h)))
       "prenorm" : h += mixer(pre_m(h));         h += ffn(pre_f(h))
+      "parallel": x = pre_m(h);  h += mixer(x) + ffn(x)      (``ffn`` may be None)
     ``norms`` holds the roles pre_mixer, post_mixer, pre_ffn, post_ffn that the
     arrangement uses.
     """
@@ -175,6 +245,7 @@ class LayerCall:
     """
     layer: int
     cache_of: Optional[int] = None
+    add_embedding: bool = False      # the embedding's output is added to the stream right before this entry
 
 
 @dataclass(frozen=True)

@@ -16,13 +16,18 @@
 
 #define AP_MAX_HD 256
 
+// MAXD: the most channels a head's queries, keys and values have (256, or 1024 for the wide rows
+// of a latent cache).  sinks (may be null): float [nh], exp(sink) joins a head's denominator with
+// no key and no value.  v_in_k: a value is the first vd channels of its key (no value cache).
+template <int MAXD>
 __global__ __launch_bounds__(64) void attention_plain_kernel(
     const act_t* __restrict__ q, int q_stride, const act_t* __restrict__ kcache,
     const act_t* __restrict__ vcache, const int* __restrict__ block_table, int max_blocks,
     const int* __restrict__ req_of_token, const int* __restrict__ positions,
     act_t* __restrict__ out, int nh, int nkv, int hd, int vd, int bs, float scale, float softcap,
-    int window, int v_transposed, const float* __restrict__ v_freq, int v_interleaved) {
-  __shared__ float sq[AP_MAX_HD];
+    int window, int v_transposed, const float* __restrict__ v_freq, int v_interleaved,
+    const float* __restrict__ sinks, int v_in_k) {
+  __shared__ float sq[MAXD];
   __shared__ float sp[64];
   __shared__ int spage[64];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -41,7 +46,7 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
   __syncthreads();
 
   float m = -INFINITY, l = 0.f;
-  float acc[AP_MAX_HD / 64] = {};
+  float acc[MAXD / 64] = {};
   for (int j0 = (lo / 64) * 64; j0 <= pos; j0 += 64) {
     const int j = j0 + lane;
     const bool valid = j >= lo && j <= pos;
@@ -65,27 +70,39 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
     spage[lane] = page;
     __syncthreads();
 #pragma unroll
-    for (int c = 0; c < AP_MAX_HD / 64; c++) {
+    for (int c = 0; c < MAXD / 64; c++) {
       const int d = lane + c * 64;
       if (d < vd) {
         float a = acc[c] * corr;
         for (int jj = 0; jj < 64; jj++) {
           const int pg = spage[jj];
           if (pg < 0) continue;
-          const size_t head_base = ((size_t)pg * nkv + kvh) * bs * vd;
           const size_t off = (j0 + jj) % bs;
-          const act_t v = v_transposed ? vcache[head_base + (size_t)d * bs + off]
-                                       : vcache[head_base + off * vd + d];
+          act_t v;
+          if (v_in_k) {
+            v = kcache[(((size_t)pg * nkv + kvh) * bs + off) * hd + d];
+          } else {
+            const size_t head_base = ((size_t)pg * nkv + kvh) * bs * vd;
+            v = v_transposed ? vcache[head_base + (size_t)d * bs + off] : vcache[head_base + off * vd + d];
+          }
           a = fmaf(sp[jj], to_f32(v), a);
         }
         acc[c] = a;
       }
     }
   }
+  if (sinks != nullptr) {
+    const float sk = sinks[h];
+    const float m_new = fmaxf(m, sk);
+    const float corr = expf(m - m_new);
+    l = l * corr + expf(sk - m_new);
+#pragma unroll
+    for (int c = 0; c < MAXD / 64; c++) acc[c] *= corr;
+  }
   const float inv = 1.f / l;
   if (v_freq == nullptr) {
 #pragma unroll
-    for (int c = 0; c < AP_MAX_HD / 64; c++) {
+    for (int c = 0; c < MAXD / 64; c++) {
       const int d = lane + c * 64;
       if (d < vd) o[d] = from_f32<act_t>(acc[c] * inv);
     }
@@ -95,7 +112,7 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
   // by the query's position, pair m by -pos * v_freq[m]
   __syncthreads();
 #pragma unroll
-  for (int c = 0; c < AP_MAX_HD / 64; c++) {
+  for (int c = 0; c < MAXD / 64; c++) {
     const int d = lane + c * 64;
     if (d < vd) sq[d] = acc[c] * inv;
   }
@@ -115,25 +132,45 @@ __global__ __launch_bounds__(64) void attention_plain_kernel(
 // cached as [page][kv head][hd][bs] instead of [page][kv head][bs][hd].
 // hd: the size of a head's queries and keys; vd: of its values (the output's too).  v_freq (may
 // be null): float [vd / 2], values are cached turned by their positions and the output is turned back.
+// sinks (may be null): float [nh].  v_in_k: values are the first vd channels of the keys.
+extern "C" int zk_attention_plain_sink(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                       const int* block_table, int max_blocks, const int* req_of_token,
+                                       const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
+                                       int bs, float scale, float softcap, int window, int v_transposed,
+                                       const float* v_freq, int v_interleaved, const float* sinks, int v_in_k,
+                                       void* stream) {
+  ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && bs > 0 && max_blocks > 0,
+             "zk_attention_plain: bad sizes");
+  ZK_REQUIRE(vd <= 1024 && (v_freq == nullptr || vd % 2 == 0), "zk_attention_plain: value size above 1024, or odd with a rotation");
+  ZK_REQUIRE(nh % nkv == 0, "zk_attention_plain: heads must be a multiple of kv heads");
+  ZK_REQUIRE(hd <= 1024, "zk_attention_plain: head_dim above 1024 is not supported");
+  ZK_REQUIRE(nh <= 65535, "zk_attention_plain: too many heads");
+  ZK_REQUIRE(q_stride >= nh * hd, "zk_attention_plain: q row stride too small");
+  ZK_REQUIRE(!v_in_k || (vd <= hd && !v_transposed), "zk_attention_plain: values inside keys are no wider than the keys");
+  if (T == 0) return 0;
+  dim3 grid(T, nh);
+  if (hd <= AP_MAX_HD && vd <= AP_MAX_HD)
+    attention_plain_kernel<AP_MAX_HD><<<grid, 64, 0, (hipStream_t)stream>>>(
+        (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
+        req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
+        v_interleaved, sinks, v_in_k);
+  else
+    attention_plain_kernel<1024><<<grid, 64, 0, (hipStream_t)stream>>>(
+        (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
+        req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
+        v_interleaved, sinks, v_in_k);
+  return zk_launch_status("zk_attention_plain");
+}
+
 extern "C" int zk_attention_plain_ext(const void* q, int q_stride, const void* kcache, const void* vcache,
                                       const int* block_table, int max_blocks, const int* req_of_token,
                                       const int* positions, void* out, int T, int nh, int nkv, int hd, int vd,
                                       int bs, float scale, float softcap, int window, int v_transposed,
                                       const float* v_freq, int v_interleaved, void* stream) {
-  ZK_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && vd > 0 && bs > 0 && max_blocks > 0,
-             "zk_attention_plain: bad sizes");
-  ZK_REQUIRE(vd <= AP_MAX_HD && (v_freq == nullptr || vd % 2 == 0), "zk_attention_plain: value size above 256, or odd with a rotation");
-  ZK_REQUIRE(nh % nkv == 0, "zk_attention_plain: heads must be a multiple of kv heads");
-  ZK_REQUIRE(hd <= AP_MAX_HD, "zk_attention_plain: head_dim above 256 is not supported");
-  ZK_REQUIRE(nh <= 65535, "zk_attention_plain: too many heads");
-  ZK_REQUIRE(q_stride >= nh * hd, "zk_attention_plain: q row stride too small");
-  if (T == 0) return 0;
-  dim3 grid(T, nh);
-  attention_plain_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(
-      (const act_t*)q, q_stride, (const act_t*)kcache, (const act_t*)vcache, block_table, max_blocks,
-      req_of_token, positions, (act_t*)out, nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq,
-      v_interleaved);
-  return zk_launch_status("zk_attention_plain");
+  ZK_REQUIRE(hd <= AP_MAX_HD && vd <= AP_MAX_HD, "zk_attention_plain: head_dim above 256 is not supported");
+  return zk_attention_plain_sink(q, q_stride, kcache, vcache, block_table, max_blocks, req_of_token, positions, out, T,
+                                 nh, nkv, hd, vd, bs, scale, softcap, window, v_transposed, v_freq, v_interleaved,
+                                 nullptr, 0, stream);
 }
 
 extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcache, const void* vcache,
@@ -147,6 +184,9 @@ extern "C" int zk_attention_plain(const void* q, int q_stride, const void* kcach
 
 #include "packed_call.h"
 extern "C" int zk_steplist_register(const char* name, int nargs, void* fn);
+static const int attention_plain_sink_entered = zk_steplist_register(
+    "zk_attention_plain_sink", zk_packed::Call<zk_attention_plain_sink>::nargs,
+    (void*)zk_packed::Call<zk_attention_plain_sink>::call);
 static const int attention_plain_ext_entered = zk_steplist_register(
     "zk_attention_plain_ext", zk_packed::Call<zk_attention_plain_ext>::nargs,
     (void*)zk_packed::Call<zk_attention_plain_ext>::call);

@@ -22,7 +22,8 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
     act_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slot_map,
     const float* __restrict__ q_gain, const float* __restrict__ k_gain, const float* __restrict__ head_scale, float eps,
     const float* __restrict__ inv_freq, int rot_dims, const float* __restrict__ v_freq, int v_interleaved,
-    act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh, int nkv, int D, int E, int bs, int v_transposed) {
+    act_t* __restrict__ kcache, act_t* __restrict__ vcache, int nh, int nkv, int D, int E, int bs, int v_transposed,
+    const float* __restrict__ bias, float rot_scale, int qk_interleaved) {
   __shared__ float buf[HP_MAX];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
@@ -35,7 +36,8 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
   if (kind != 0 && slot < 0) return;
   float sum = 0.f;
   for (int d = lane; d < size; d += 64) {
-    const float x = to_f32(qkv[at + d]);
+    float x = to_f32(qkv[at + d]);
+    if (bias) x += bias[at - (size_t)t * width + d];
     buf[d] = x;
     sum = fmaf(x, x, sum);
   }
@@ -53,11 +55,16 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
   // rotation: every lane takes whole pairs, so nothing is read after another lane wrote it
   const float* freq = kind == 2 ? v_freq : inv_freq;
   const int dims = kind == 2 ? (v_freq ? E : 0) : (inv_freq ? rot_dims : 0);
-  const bool inter = kind == 2 && v_interleaved;
+  const bool inter = kind == 2 ? v_interleaved : qk_interleaved;
+  const float mag = kind == 2 ? 1.0f : rot_scale;
   const int half = dims / 2;
   for (int m = lane; m < half; m += 64) {
     float sn, cs, ra, rb;
     sincosf((float)pos * freq[m], &sn, &cs);
+    if (mag != 1.0f) {
+      sn *= mag;
+      cs *= mag;
+    }
     const int ia = inter ? 2 * m : m, ib = inter ? 2 * m + 1 : m + half;
     rotate_pair(buf[ia], buf[ib], sn, cs, ra, rb);
     buf[ia] = ra;
@@ -83,10 +90,14 @@ __global__ __launch_bounds__(64) void head_prep_kernel(
 
 // nkv: key/value heads held in the rows (0 for a mixer that stores none).  q_gain, k_gain,
 // head_scale, inv_freq, v_freq may each be null (the step it stands for is then left out).
-extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
-                            const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
-                            int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
-                            int nh, int nkv, int D, int E, int bs, int v_transposed, void* stream) {
+// bias (may be null): float, one per channel of a row, added before anything else.  rot_scale:
+// multiplies the sines and cosines of queries and keys.  qk_interleaved: their pairs are
+// (2i, 2i + 1) instead of (i, i + rot_dims / 2).
+extern "C" int zk_head_prep_ext(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
+                                const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
+                                int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
+                                int nh, int nkv, int D, int E, int bs, int v_transposed, const float* bias,
+                                float rot_scale, int qk_interleaved, void* stream) {
   ZK_REQUIRE(T >= 0 && nh > 0 && nkv >= 0 && D > 0 && E > 0 && bs > 0, "zk_head_prep: bad sizes");
   ZK_REQUIRE(D <= HP_MAX && E <= HP_MAX, "zk_head_prep: heads of more than 256 channels are not supported");
   ZK_REQUIRE(inv_freq == nullptr || (rot_dims % 2 == 0 && rot_dims >= 0 && rot_dims <= D),
@@ -98,9 +109,20 @@ extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map
   dim3 grid(T, nh + 2 * nkv);
   head_prep_kernel<<<grid, 64, 0, (hipStream_t)stream>>>((act_t*)qkv, positions, slot_map, q_gain, k_gain, head_scale, eps,
                                                          inv_freq, rot_dims, v_freq, v_interleaved, (act_t*)kcache,
-                                                         (act_t*)vcache, nh, nkv, D, E, bs, v_transposed);
+                                                         (act_t*)vcache, nh, nkv, D, E, bs, v_transposed, bias, rot_scale,
+                                                         qk_interleaved);
   return zk_launch_status("zk_head_prep");
+}
+
+extern "C" int zk_head_prep(void* qkv, const int* positions, const int* slot_map, const float* q_gain,
+                            const float* k_gain, const float* head_scale, float eps, const float* inv_freq,
+                            int rot_dims, const float* v_freq, int v_interleaved, void* kcache, void* vcache, int T,
+                            int nh, int nkv, int D, int E, int bs, int v_transposed, void* stream) {
+  return zk_head_prep_ext(qkv, positions, slot_map, q_gain, k_gain, head_scale, eps, inv_freq, rot_dims, v_freq,
+                          v_interleaved, kcache, vcache, T, nh, nkv, D, E, bs, v_transposed, nullptr, 1.0f, 0, stream);
 }
 
 static const int head_prep_entered =
     zk_steplist_register("zk_head_prep", zk_packed::Call<zk_head_prep>::nargs, (void*)zk_packed::Call<zk_head_prep>::call);
+static const int head_prep_ext_entered = zk_steplist_register(
+    "zk_head_prep_ext", zk_packed::Call<zk_head_prep_ext>::nargs, (void*)zk_packed::Call<zk_head_prep_ext>::call);

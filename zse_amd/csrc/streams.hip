@@ -137,27 +137,30 @@ template <bool RENEW>
 __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __restrict__ w, float* __restrict__ state,
                                   int slot_words, int offset_words, const int* __restrict__ positions,
                                   const int* __restrict__ req_of_token, const int* __restrict__ q_start,
-                                  const int* __restrict__ slot_of_req, act_t* __restrict__ out, int W, int taps) {
+                                  const int* __restrict__ slot_of_req, act_t* __restrict__ out, int W, int taps,
+                                  int ld_in, int ld_out, int residual, int act) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= W) return;
   if (positions[t] < 0) {             // a padding row of a captured step
-    out[(size_t)t * W + c] = from_f32<act_t>(0.f);
+    out[(size_t)t * ld_out + c] = from_f32<act_t>(0.f);
     return;
   }
   const int r = req_of_token[t];
   const int before = t - q_start[r];      // rows of this step in front of t that belong to the same request
   float* st = state + (size_t)slot_of_req[r] * slot_words + offset_words;
-  const float x = to_f32(h[(size_t)t * W + c]);
+  const float x = to_f32(h[(size_t)t * ld_in + c]);
   float acc = 0.f;
   for (int j = 0; j < taps; j++) {
     const int back = taps - 1 - j;
     float v;
-    if (back <= before) v = to_f32(h[(size_t)(t - back) * W + c]);
+    if (back <= before) v = to_f32(h[(size_t)(t - back) * ld_in + c]);
     else v = st[(size_t)(back - before - 1) * W + c];      // state row a holds the row a + 1 places before the step
     acc = fmaf(w[(size_t)c * taps + j], v, acc);
   }
-  out[(size_t)t * W + c] = from_f32<act_t>(x + acc);
+  if (residual) acc = x + acc;
+  if (act == 1) acc = acc / (1.0f + expf(-acc));      // silu
+  out[(size_t)t * ld_out + c] = from_f32<act_t>(acc);
   if (RENEW) {
     for (int a = taps - 2; a > 0; a--) st[(size_t)a * W + c] = st[(size_t)(a - 1) * W + c];
     if (taps > 1) st[c] = x;
@@ -166,7 +169,7 @@ __global__ void short_conv_kernel(const act_t* __restrict__ h, const float* __re
 
 __global__ void short_conv_state_kernel(const act_t* __restrict__ h, float* __restrict__ state, int slot_words,
                                         int offset_words, const int* __restrict__ q_start,
-                                        const int* __restrict__ slot_of_req, int W, int taps) {
+                                        const int* __restrict__ slot_of_req, int W, int taps, int ld_in) {
   const int r = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= W) return;
@@ -178,7 +181,7 @@ __global__ void short_conv_state_kernel(const act_t* __restrict__ h, float* __re
   // rows, or an older state row moved back by n; from the oldest on, so nothing is read after
   // it was overwritten
   for (int a = taps - 2; a >= 0; a--) {
-    const float v = a < n ? to_f32(h[(size_t)(t1 - 1 - a) * W + c]) : st[(size_t)(a - n) * W + c];
+    const float v = a < n ? to_f32(h[(size_t)(t1 - 1 - a) * ld_in + c]) : st[(size_t)(a - n) * W + c];
     st[(size_t)a * W + c] = v;
   }
 }
@@ -249,12 +252,15 @@ int zk_streams_step(float* xs, int S, const void* y, int y_parts, const float* w
   return zk_launch_status("zk_streams_step");
 }
 
-// h, out: [T, W] activations; w: float [W, taps]; the state of request r is taps - 1 float rows
-// of W at state[slot_of_req[r] * slot_words + offset_words].
-int zk_short_conv(const void* h, const float* w, const float* state, int slot_words, int offset_words,
-                  const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
-                  void* out, int T, int W, int taps, void* stream) {
+// h: [T, ld_in] activations, out: [T, ld_out], of which the first W channels take part; w: float
+// [W, taps]; the state of request r is taps - 1 float rows of W at
+// state[slot_of_req[r] * slot_words + offset_words].  residual: the input is added to the sum;
+// act: 0 none, 1 silu (after the sum).
+int zk_short_conv_ext(const void* h, int ld_in, const float* w, const float* state, int slot_words, int offset_words,
+                      const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                      void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
   ZK_REQUIRE(T >= 0 && T <= 65535 * 16 && W > 0 && taps >= 1, "zk_short_conv: bad sizes");
+  ZK_REQUIRE(ld_in >= W && ld_out >= W && (act == 0 || act == 1), "zk_short_conv: bad strides or activation");
   ZK_REQUIRE(taps == 1 || (state != nullptr && slot_words >= offset_words + (taps - 1) * W),
              "zk_short_conv: the state does not fit its slot");
   if (T == 0) return 0;
@@ -262,35 +268,56 @@ int zk_short_conv(const void* h, const float* w, const float* state, int slot_wo
   dim3 grid((W + 255) / 256, T);
   short_conv_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, (float*)state, slot_words, offset_words,
                                                                   positions, req_of_token, q_start, slot_of_req,
-                                                                  (act_t*)out, W, taps);
+                                                                  (act_t*)out, W, taps, ld_in, ld_out, residual, act);
   return zk_launch_status("zk_short_conv");
+}
+
+int zk_short_conv(const void* h, const float* w, const float* state, int slot_words, int offset_words,
+                  const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                  void* out, int T, int W, int taps, void* stream) {
+  return zk_short_conv_ext(h, W, w, state, slot_words, offset_words, positions, req_of_token, q_start, slot_of_req, out, W,
+                           T, W, taps, 1, 0, stream);
 }
 
 // The convolution and the renewal of the state in one launch, for steps in which every request
 // brings exactly one token (T rows, T requests).
-int zk_short_conv_token(const void* h, const float* w, float* state, int slot_words, int offset_words,
-                        const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
-                        void* out, int T, int W, int taps, void* stream) {
+int zk_short_conv_token_ext(const void* h, int ld_in, const float* w, float* state, int slot_words, int offset_words,
+                            const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                            void* out, int ld_out, int T, int W, int taps, int residual, int act, void* stream) {
   ZK_REQUIRE(T >= 0 && T <= 65535 && W > 0 && taps >= 1, "zk_short_conv_token: bad sizes");
+  ZK_REQUIRE(ld_in >= W && ld_out >= W && (act == 0 || act == 1), "zk_short_conv_token: bad strides or activation");
   ZK_REQUIRE(taps == 1 || (state != nullptr && slot_words >= offset_words + (taps - 1) * W),
              "zk_short_conv_token: the state does not fit its slot");
   if (T == 0) return 0;
   dim3 grid((W + 255) / 256, T);
   short_conv_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, w, state, slot_words, offset_words, positions,
-                                                                 req_of_token, q_start, slot_of_req, (act_t*)out, W, taps);
+                                                                 req_of_token, q_start, slot_of_req, (act_t*)out, W, taps,
+                                                                 ld_in, ld_out, residual, act);
   return zk_launch_status("zk_short_conv_token");
 }
 
-int zk_short_conv_state(const void* h, float* state, int slot_words, int offset_words, const int* q_start,
-                        const int* slot_of_req, int R, int W, int taps, void* stream) {
-  ZK_REQUIRE(R >= 0 && R <= 65535 && W > 0 && taps >= 1, "zk_short_conv_state: bad sizes");
+int zk_short_conv_token(const void* h, const float* w, float* state, int slot_words, int offset_words,
+                        const int* positions, const int* req_of_token, const int* q_start, const int* slot_of_req,
+                        void* out, int T, int W, int taps, void* stream) {
+  return zk_short_conv_token_ext(h, W, w, state, slot_words, offset_words, positions, req_of_token, q_start, slot_of_req,
+                                 out, W, T, W, taps, 1, 0, stream);
+}
+
+int zk_short_conv_state_ext(const void* h, int ld_in, float* state, int slot_words, int offset_words, const int* q_start,
+                            const int* slot_of_req, int R, int W, int taps, void* stream) {
+  ZK_REQUIRE(R >= 0 && R <= 65535 && W > 0 && taps >= 1 && ld_in >= W, "zk_short_conv_state: bad sizes");
   if (R == 0 || taps == 1) return 0;
   ZK_REQUIRE(state != nullptr && slot_words >= offset_words + (taps - 1) * W,
              "zk_short_conv_state: the state does not fit its slot");
   dim3 grid((W + 255) / 256, R);
   short_conv_state_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)h, state, slot_words, offset_words,
-                                                                 q_start, slot_of_req, W, taps);
+                                                                 q_start, slot_of_req, W, taps, ld_in);
   return zk_launch_status("zk_short_conv_state");
+}
+
+int zk_short_conv_state(const void* h, float* state, int slot_words, int offset_words, const int* q_start,
+                        const int* slot_of_req, int R, int W, int taps, void* stream) {
+  return zk_short_conv_state_ext(h, W, state, slot_words, offset_words, q_start, slot_of_req, R, W, taps, stream);
 }
 
 // x: [T, heads * size] activations; pair m of a head (m, m + size/2; interleaved: 2m, 2m + 1) is
@@ -310,4 +337,7 @@ ZK_ENTER(zk_streams_step)
 ZK_ENTER(zk_short_conv)
 ZK_ENTER(zk_short_conv_token)
 ZK_ENTER(zk_short_conv_state)
+ZK_ENTER(zk_short_conv_ext)
+ZK_ENTER(zk_short_conv_token_ext)
+ZK_ENTER(zk_short_conv_state_ext)
 ZK_ENTER(zk_rotate_heads)

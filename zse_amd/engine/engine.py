@@ -107,7 +107,8 @@ class Engine:
         groups = group_needs(needs)
         item = 2 if self.dtype == "bfloat16" else 4
         def bytes_per_page(g):
-            return sum(needs[c].num_kv_heads * (needs[c].head_dim + (needs[c].value_dim or needs[c].head_dim))
+            return sum(needs[c].num_kv_heads * (needs[c].head_dim + (0 if getattr(needs[c], "values_in_keys", False)
+                                                              else (needs[c].value_dim or needs[c].head_dim)))
                        for c in g.calls) * item * block_size
         def windowed_pages(g):
             per_request = -(-(g.window + step_tokens) // block_size) + 2

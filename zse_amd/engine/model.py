@@ -105,8 +105,24 @@ class Model:
         for need in self.cache_needs():
             if isinstance(need, PagedKV):
                 seen = min(context, need.window) if need.window else context
-                total += need.num_kv_heads * (need.head_dim + (need.value_dim or need.head_dim)) * seen * itemsize
+                vd = 0 if getattr(need, "values_in_keys", False) else (need.value_dim or need.head_dim)
+                total += need.num_kv_heads * (need.head_dim + vd) * seen * itemsize
         return total
+
+    @staticmethod
+    def _add_embedding(ctx, h: Tensor, first: Tensor, blk, out: Tensor):
+        """h += the embedding's output; returns the block's entry norm of the new stream where the
+        joining kernel can make it in the same launch (an RMS norm), else None."""
+        from ..parts.norm import RMSNorm
+        norm = blk.entry_norm() if hasattr(blk, "entry_norm") else None
+        T, H = h.shape
+        if isinstance(norm, RMSNorm):
+            ns = norm.spec
+            ctx.k.zk_sum_norm(h.ptr, first.ptr, 1, None, 0, None, norm.weight.ptr, float(ns.eps), int(ns.unit_offset),
+                              out.ptr, T, H, ctx.stream)
+            return Tensor(out.ptr, (T, H), ctx.dtype, out.owner)
+        ctx.k.zk_sum_norm(h.ptr, first.ptr, 1, None, 0, None, None, 0.0, 0, None, T, H, ctx.stream)
+        return None
 
     def forward(self, ctx, caches: List[CallCache], logit_rows, n_rows: int, logits: Tensor, pick=None):
         """Run the step's tokens through every entry of the order; write float
@@ -119,12 +135,20 @@ class Model:
         # its output alternates between two buffers that outlive a layer's own
         T, H = h.shape
         handoff = [ctx.alloc((T, H)), ctx.alloc((T, H))]
+        # an order that adds the embedding's output to the stream again keeps a copy of it
+        again = any(getattr(c, "add_embedding", False) for c in order)
+        # (gathered a second time: a launch like any other, which a captured or written-down step repeats)
+        first = self.embedding.forward(ctx) if again else None
         x = None
         base = ctx.arena.mark()
         for i, call in enumerate(order):
             cache = caches[i] if caches[i].shared else caches[call.cache_of if call.cache_of is not None else i]
             blk = self.blocks[call.layer]
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
+            if nxt is not None and getattr(order[i + 1], "add_embedding", False):
+                nxt = None           # the stream changes between the two entries: the next one norms it itself
+            if getattr(call, "add_embedding", False):
+                x = self._add_embedding(ctx, h, first, blk, handoff[(i + 1) % 2])
             if hasattr(blk, "entry_norm"):
                 next_norm = nxt.entry_norm() if nxt is not None and hasattr(nxt, "entry_norm") else None
                 x = blk.forward(ctx, h, cache, x_in=x, next_norm=next_norm, x_out=handoff[i % 2])

@@ -195,7 +195,8 @@ class StepRunner:
                 shape = (pages, need.num_kv_heads, self.page_size, vd)
                 if cc.v_transposed:
                     shape = (pages, need.num_kv_heads, vd, self.page_size)
-                cc.v = rt.zeros(shape, self.dtype)
+                # values that are part of the keys have no slab of their own
+                cc.v = cc.k if getattr(need, "values_in_keys", False) else rt.zeros(shape, self.dtype)
             elif isinstance(need, StateNeed):
                 cc.state_offset = slot_bytes
                 cc.state_bytes = int(need.nbytes)
@@ -219,7 +220,8 @@ class StepRunner:
         # clears a page in all of them
         self._slabs = []
         for gid in range(len(groups)):
-            ts = [t for cc in self.caches if cc.group == gid and cc.k is not None and not cc.shared for t in (cc.k, cc.v)]
+            ts = [t for cc in self.caches if cc.group == gid and cc.k is not None and not cc.shared
+                  for t in ((cc.k,) if cc.v is cc.k else (cc.k, cc.v))]
             ptrs = rt.upload(np.array([t.ptr for t in ts], dtype=np.uint64).view(np.float64), "float64")
             sizes = rt.upload(np.array([t.nbytes // t.shape[0] for t in ts], dtype=np.uint64).view(np.float64), "float64")
             self._slabs.append((ptrs, sizes, len(ts)))
@@ -285,7 +287,7 @@ class StepRunner:
         return 4 * T + (R + 1) + 4 * R + G * (T + R * self.max_blocks) + 64
 
     def cache_bytes(self) -> int:
-        return sum(c.k.nbytes + c.v.nbytes for c in self.caches if c.k is not None and not c.shared)
+        return sum(c.k.nbytes + (0 if c.v is c.k else c.v.nbytes) for c in self.caches if c.k is not None and not c.shared)
 
     # ------------------------------------------------------------------ requests
     def _clear_slot(self, req, slot: int) -> None:

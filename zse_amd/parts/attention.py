@@ -40,8 +40,13 @@ class PagedAttention(Part):
         self.q_norm_name, self.k_norm_name = getattr(s, "q_norm", None), getattr(s, "k_norm", None)
         self.head_scale_name = getattr(s, "head_scale", None)
         self.value_base = getattr(s, "value_rotation", None)
+        self.bias_names = dict(getattr(s, "biases", None) or {})
+        self.rot_scale = float(self.position.magnitude()) if hasattr(self.position, "magnitude") else 1.0
+        self.rot_interleaved = bool(getattr(self.position, "interleaved", False))
         self.general = bool(self.value_dim != s.head_dim or self.q_norm_name or self.k_norm_name or
-                            self.head_scale_name or self.value_base)
+                            self.head_scale_name or self.value_base or self.bias_names or
+                            self.rot_scale != 1.0 or self.rot_interleaved)
+        self.in_bias = self.o_bias = None
         if self.value_dim > 256:
             raise ValueError(f"value_dim up to 256, got {self.value_dim}")
         if self.value_base and self.value_dim % 2:
@@ -60,8 +65,14 @@ class PagedAttention(Part):
             out.append(TensorReq(self.q_norm_name, (s.head_dim,), ROLE_GAIN))
         if self.head_scale_name:
             out.append(TensorReq(self.head_scale_name, (s.num_heads,), ROLE_GAIN))
+        for role, rows in (("q", s.num_heads * s.head_dim), ("o", s.hidden_size)):
+            if role in self.bias_names:
+                out.append(TensorReq(self.bias_names[role], (rows,), ROLE_GAIN))
         if self.shared_kv:
             return out
+        for role, rows in (("k", s.num_kv_heads * s.head_dim), ("v", s.num_kv_heads * self.value_dim)):
+            if role in self.bias_names:
+                out.append(TensorReq(self.bias_names[role], (rows,), ROLE_GAIN))
         out += [TensorReq(s.names["k"], (s.num_kv_heads * s.head_dim, s.hidden_size)),
                 TensorReq(s.names["v"], (s.num_kv_heads * self.value_dim, s.hidden_size))]
         if self.k_norm_name:
@@ -82,6 +93,13 @@ class PagedAttention(Part):
             self.k_gain = weights.vector(self.k_norm_name)
         if self.head_scale_name:
             self.head_scale = weights.vector(self.head_scale_name)
+        roles = ("q",) if self.shared_kv else ("q", "k", "v")
+        if any(r in self.bias_names for r in roles):
+            if not all(r in self.bias_names for r in roles):
+                raise ValueError("biases on the projections: all of q, k, v or none")
+            self.in_bias = weights.vectors([self.bias_names[r] for r in roles])
+        if "o" in self.bias_names:
+            self.o_bias = weights.vector(self.bias_names["o"])
         if self.value_base:
             m = np.arange(self.value_dim // 2, dtype=np.float64)
             self.value_freq = rt.upload(np.power(float(self.value_base), -2.0 * m / self.value_dim).astype(np.float32))
@@ -153,10 +171,12 @@ class PagedAttention(Part):
         ptr = lambda t: t.ptr if t is not None else None
         vfreq = ptr(self.value_freq)
         inter = 1 if getattr(s, "value_pairs_interleaved", False) else 0
-        k.zk_head_prep(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain), ptr(self.k_gain),
-                       ptr(self.head_scale), float(s.norm_eps), tables[0].ptr if tables is not None else None,
-                       tables[1] if tables is not None else 0, vfreq, inter, cache.k.ptr, cache.v.ptr, T, nh, n_store,
-                       hd, vd, g.page_size, 1 if cache.v_transposed else 0, ctx.stream)
+        k.zk_head_prep_ext(qkv.ptr, ctx.positions, None if self.shared_kv else g.slot_map, ptr(self.q_gain),
+                           ptr(self.k_gain), ptr(self.head_scale), float(s.norm_eps),
+                           tables[0].ptr if tables is not None else None, tables[1] if tables is not None else 0, vfreq,
+                           inter, cache.k.ptr, cache.v.ptr, T, nh, n_store, hd, vd, g.page_size,
+                           1 if cache.v_transposed else 0, ptr(self.in_bias), self.rot_scale,
+                           1 if self.rot_interleaved else 0, ctx.stream)
         o = ctx.alloc((T, nh * vd))
         cap = float(s.softcap) if s.softcap else 0.0
         win = int(s.window) if s.window else 0
@@ -171,7 +191,13 @@ class PagedAttention(Part):
             k.zk_attention_plain_ext(qkv.ptr, width, cache.k.ptr, cache.v.ptr, g.block_table, g.max_blocks,
                                      ctx.req_of_token, ctx.positions, o.ptr, T, nh, nkv, hd, vd, g.page_size, s.scale,
                                      cap, win, 1 if cache.v_transposed else 0, vfreq, inter, ctx.stream)
-        return linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
+        y = linear(ctx, o, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self if self.o_bias is None else None)
+        if self.o_bias is not None:
+            if getattr(ctx, "bias_welcome", None) is self:
+                ctx.result_bias = self.o_bias          # the block's joining kernel adds it
+            else:
+                k.zk_add_bias(y.ptr, self.o_bias.ptr, T, s.hidden_size, ctx.stream)
+        return y
 
     def forward(self, ctx, x: Tensor, cache) -> Tensor:
         if self.general:

@@ -48,6 +48,7 @@ class PagedKV:
     head_dim: int
     window: Optional[int]
     value_dim: Optional[int] = None     # size of a head's values where it differs from its keys'
+    values_in_keys: bool = False        # a value is the first value_dim channels of its key: no value slab is kept
 
 
 @dataclass(frozen=True)

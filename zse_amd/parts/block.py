@@ -86,4 +86,54 @@ class Block(Part):
         return self._join(ctx, m, n.get("post_ffn"), h, next_norm, x_out)
 
 
-register_part("block", "block", Block)
+class ParallelBlock(Part):
+    """x = norm(h); h += mixer(x) + ffn(x): one norm, both sublayers read it, and their results
+    are summed before they join the float stream (``ffn`` None: the mixer alone).  One kernel
+    does the sum, the mixer's output bias if it has one, the residual sum and the norm of
+    whatever runs next."""
+    graph_safe = True      # its launches take what changes from step to step from device memory alone
+
+    def __init__(self, spec):
+        self.spec = spec
+        if "pre_mixer" not in spec.norms:
+            raise ValueError("a parallel block needs the norm pre_mixer")
+        self.norms = {"pre_mixer": build_part("norm", spec.norms["pre_mixer"])}
+        self.mixer = build_part("mixer", spec.mixer)
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+
+    def children(self):
+        return list(self.norms.values()) + [self.mixer] + ([self.ffn] if self.ffn is not None else [])
+
+    def entry_norm(self):
+        return self.norms["pre_mixer"]
+
+    def forward(self, ctx, h: Tensor, cache, x_in: Tensor = None, next_norm=None, x_out: Tensor = None):
+        T, H = h.shape
+        x = x_in if x_in is not None else self.norms["pre_mixer"].forward(ctx, h)
+        # the mixer's result has to outlive the feed-forward's products: no partial sums in the
+        # products' shared workspace; its output bias is added by the joining kernel
+        ctx.sums_welcome, ctx.bias_welcome, ctx.result_bias = None, self.mixer, None
+        a = self.mixer.forward(ctx, x, cache)
+        bias, ctx.bias_welcome, ctx.result_bias = ctx.result_bias, None, None
+        m = None
+        if self.ffn is not None:
+            ctx.sums_welcome = self.ffn
+            m = self.ffn.forward(ctx, x)
+            ctx.sums_welcome = None
+        ns = next_norm.spec if isinstance(next_norm, RMSNorm) else None
+        out = None
+        if ns is not None:
+            out = ctx.alloc((T, H)) if x_out is None else Tensor(x_out.ptr, (T, H), ctx.dtype, x_out.owner)
+        planes = lambda t: t.shape[0] if (t is not None and t.layout == "parts") else 0
+        ctx.k.zk_sum_norm(h.ptr, a.ptr, planes(a), m.ptr if m is not None else None, planes(m),
+                          bias.ptr if bias is not None else None, next_norm.weight.ptr if ns is not None else None,
+                          float(ns.eps) if ns is not None else 0.0, int(ns.unit_offset) if ns is not None else 0,
+                          out.ptr if out is not None else None, T, H, ctx.stream)
+        return out
+
+
+def _block(spec):
+    return ParallelBlock(spec) if spec.arrangement == "parallel" else Block(spec)
+
+
+register_part("block", "block", _block)

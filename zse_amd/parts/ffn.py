@@ -10,19 +10,22 @@ from __future__ import annotations
 
 from typing import List
 
-from ..runtime.device import Tensor
-from .base import Part, TensorReq, register_part
+from ..runtime.device import BF16, F32, I32, Tensor
+from .base import Part, TensorReq, build_part, register_part
 from .ops import linear, tuned_gemm
 
 ACTIVATION_CODES = {"gelu_tanh": 0, "silu": 1, "relu": 2}
+CLAMPED = "clamped_swiglu"     # g = min(gate, limit), u = clamp(up, +-limit): g sigmoid(1.702 g) (u + 1)
 
 
 class GatedMLP(Part):
     graph_safe = True      # its launches take what changes from step to step from device memory alone
 
     def __init__(self, spec):
-        if spec.activation not in ACTIVATION_CODES:
-            raise ValueError(f"activation must be one of {sorted(ACTIVATION_CODES)}, got {spec.activation!r}")
+        if spec.activation not in ACTIVATION_CODES and spec.activation != CLAMPED:
+            raise ValueError(f"activation must be one of {sorted(ACTIVATION_CODES) + [CLAMPED]}, got {spec.activation!r}")
+        if spec.activation == CLAMPED and not (getattr(spec, "limit", None) or 0) > 0:
+            raise ValueError(f"{CLAMPED} needs a positive limit, got {getattr(spec, 'limit', None)!r}")
         self.spec = spec
         self.w_gu = self.w_down = None
 
@@ -41,9 +44,19 @@ class GatedMLP(Part):
         self.w_down = (weights.matrix([s.names["down"]], strip=True) if strip and strip(s.intermediate_size)
                        else weights.matrix([s.names["down"]]))
 
-    def forward(self, ctx, x: Tensor) -> Tensor:
+    def forward(self, ctx, x: Tensor, out: Tensor = None) -> Tensor:
+        """``out``: where the result goes (activations or float32 [T, hidden]); the product that
+        ends the layer then never hands partial sums back."""
         s = self.spec
         T, I = x.shape[0], s.intermediate_size
+        last = None if out is not None else self
+        if s.activation == CLAMPED:
+            gu = linear(ctx, x, self.w_gu, ctx.alloc((T, 2 * I)))
+            a = ctx.alloc((T, I))
+            ctx.k.zk_clamped_glu(gu.ptr, a.ptr, T, I, float(s.limit), ctx.stream)
+            return linear(ctx, a, self.w_down, out if out is not None else ctx.alloc((T, s.hidden_size)), last_of=last)
+        if out is not None:
+            raise ValueError("a result buffer of the caller's is taken by the clamped layer only")
         if tuned_gemm(ctx, s.hidden_size):
             a = linear(ctx, x, self.w_gu, ctx.alloc((T, I)), epilogue=s.activation)
             return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
@@ -53,4 +66,83 @@ class GatedMLP(Part):
         return linear(ctx, a, self.w_down, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 
+class RoutedMLP(Part):
+    """A mixture of small gated layers: sigmoid scores from a float router product, the ``top_k``
+    largest chosen on the device (the lower index among equals), the chosen scores as weights on
+    the experts' inputs, the experts' results added in the order they were chosen, a shared layer
+    on top.  Steps of few tokens read each chosen expert's rows once per (token, choice); steps of
+    many tokens sort the pairs by expert on the device and run a grouped matrix-core product.
+    Nothing comes back to the host, so steps are captured and written down like any other."""
+    graph_safe = True
+    GROUPED_FROM = 64          # (token, choice) pairs from which the grouped product is used (bfloat16)
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.activation != CLAMPED:
+            raise ValueError(f"routed experts are {CLAMPED} layers, got {s.activation!r}")
+        if not (1 <= s.top_k <= min(s.num_experts, 16)) or s.num_experts > 1024:
+            raise ValueError(f"1 to 16 of up to 1024 experts a token, got {s.top_k} of {s.num_experts}")
+        if not s.scale_input:
+            raise ValueError("routed experts take their weight on the input")
+        if not (s.limit or 0) > 0:
+            raise ValueError(f"{CLAMPED} needs a positive limit, got {s.limit!r}")
+        self.shared = build_part("ffn", s.shared) if s.shared is not None else None
+        self.w_router = self.w_gu = self.w_down = None
+
+    def children(self):
+        return [self.shared] if self.shared is not None else []
+
+    def _name(self, e: int, role: str) -> str:
+        return self.spec.expert_names.format(e=e, role=role)
+
+    def tensor_reqs(self) -> List[TensorReq]:
+        s = self.spec
+        out = [TensorReq(s.router, (s.num_experts, s.hidden_size))]
+        for e in range(s.num_experts):
+            out += [TensorReq(self._name(e, "gate"), (s.intermediate_size, s.hidden_size)),
+                    TensorReq(self._name(e, "up"), (s.intermediate_size, s.hidden_size)),
+                    TensorReq(self._name(e, "down"), (s.hidden_size, s.intermediate_size))]
+        return out
+
+    def load(self, weights, rt, dtype):
+        s = self.spec
+        self.w_router = weights.matrix([s.router])
+        # expert e: rows [e 2F, e 2F + F) its gate, the next F its up; down: rows [e W, (e + 1) W)
+        self.w_gu = weights.matrix([self._name(e, r) for e in range(s.num_experts) for r in ("gate", "up")])
+        self.w_down = weights.matrix([self._name(e, "down") for e in range(s.num_experts)])
+
+    def flops_per_token(self) -> float:
+        s = self.spec
+        return 2.0 * s.num_experts * s.hidden_size + s.top_k * 6.0 * s.intermediate_size * s.hidden_size
+
+    def forward(self, ctx, x: Tensor) -> Tensor:
+        s, k = self.spec, ctx.k
+        T, W, F, E, top = x.shape[0], s.hidden_size, s.intermediate_size, s.num_experts, s.top_k
+        logits = linear(ctx, x, self.w_router, ctx.alloc((T, E), F32))
+        ids, wts = ctx.alloc((T, top), I32), ctx.alloc((T, top), F32)
+        k.zk_moe_route(logits.ptr, ids.ptr, wts.ptr, T, E, top, ctx.stream)
+        P = 2 if self.shared is not None else 1
+        planes = ctx.alloc((P, T, W), F32)
+        y = ctx.alloc((T * top, F))
+        grouped = (ctx.dtype == BF16 and ctx.tuned and T * top >= self.GROUPED_FROM and W % 8 == 0 and F % 8 == 0
+                   and k.has("zk_moe_experts_grouped"))
+        if grouped:
+            work = ctx.alloc((E + 1 + 2 * T * top,), I32)
+            xg, rows = ctx.alloc((T * top, W)), ctx.alloc((T * top, W), F32)
+            k.zk_moe_experts_grouped(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, work.ptr, xg.ptr, y.ptr,
+                                     rows.ptr, planes.ptr, T, E, top, W, F, float(s.limit), ctx.stream)
+        else:
+            k.zk_moe_experts(x.ptr, ids.ptr, wts.ptr, self.w_gu.ptr, self.w_down.ptr, y.ptr, planes.ptr, T, top, W, F,
+                             float(s.limit), ctx.stream)
+        if self.shared is not None:
+            self.shared.forward(ctx, x, out=planes.rows(1, 2).view(T, W))
+        if getattr(ctx, "sums_welcome", None) is self:
+            # the block's joining kernel adds the planes up itself
+            return Tensor(planes.ptr, (P, T, W), F32, planes.owner, layout="parts")
+        out = ctx.alloc((T, W))
+        k.zk_planes_sum(planes.ptr, P, out.ptr, T, W, ctx.stream)
+        return out
+
+
 register_part("ffn", "gated_mlp", GatedMLP)
+register_part("ffn", "routed_mlp", RoutedMLP)

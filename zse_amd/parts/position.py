@@ -7,6 +7,8 @@ encoding must be a function of the absolute position alone.
 """
 from __future__ import annotations
 
+import math
+
 import numpy as np
 
 from ..runtime.device import Tensor
@@ -25,7 +27,27 @@ class Rotary(Part):
     def frequencies(self) -> np.ndarray:
         s = self.spec
         i = np.arange(s.rotary_dim // 2, dtype=np.float64)
-        return (1.0 / np.power(float(s.theta), 2.0 * i / s.rotary_dim)).astype(np.float32)
+        f = 1.0 / np.power(float(s.theta), 2.0 * i / s.rotary_dim)
+        scaling = getattr(s, "scaling", None)
+        if scaling is not None:
+            # pair numbers at which `fast` and `slow` turns fit into `original` positions bound a
+            # ramp; below it a frequency stays, above it is divided by the factor
+            factor, original, fast, slow = (float(v) for v in scaling)
+            at = lambda turns: s.rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(s.theta)))
+            lo = max(math.floor(at(fast)), 0)
+            hi = min(math.ceil(at(slow)), s.rotary_dim - 1)
+            ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            f = f / factor * ramp + f * (1.0 - ramp)
+        return f.astype(np.float32)
+
+    def magnitude(self) -> float:
+        """What sines and cosines are multiplied by (1 without frequency scaling)."""
+        scaling = getattr(self.spec, "scaling", None)
+        return 0.1 * math.log(float(scaling[0])) + 1.0 if scaling is not None else 1.0
+
+    @property
+    def interleaved(self) -> bool:
+        return bool(getattr(self.spec, "interleaved", False))
 
     def load(self, weights, rt, dtype):
         self.inv_freq = rt.upload(self.frequencies())

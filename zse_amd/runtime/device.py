@@ -176,6 +176,22 @@ KERNEL_SIGNATURES = {
     "zk_mlstm_chunked": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _I, _VP],
     "zk_mlstm_scan": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _F, _I, _VP],
     "zk_mlstm_finish": [_VP, _VP, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
+    "zk_short_conv_ext": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_short_conv_token_ext": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_short_conv_state_ext": [_VP, _I, _VP, _I, _I, _VP, _VP, _I, _I, _I, _VP],
+    "zk_head_prep_ext": [_VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I,
+                         _VP, _F, _I, _VP],
+    "zk_attention_plain_sink": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F,
+                                _I, _I, _VP, _I, _VP, _I, _VP],
+    "zk_delta_rule": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
+    "zk_moe_route": [_VP, _VP, _VP, _I, _I, _I, _VP],
+    "zk_moe_experts": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
+    "zk_clamped_glu": [_VP, _VP, _I, _I, _F, _VP],
+    "zk_latent_prep": [_VP, _I, _VP, _VP, _VP, _F, _VP, _F, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_heads_linear": [_VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "zk_sum_norm": [_VP, _VP, _I, _VP, _I, _VP, _VP, _F, _I, _VP, _I, _I, _VP],
+    "zk_add_bias": [_VP, _VP, _I, _I, _VP],
+    "zk_planes_sum": [_VP, _I, _VP, _I, _I, _VP],
 }
 # present only in the bf16 library
 BF16_KERNEL_SIGNATURES = {
@@ -187,6 +203,7 @@ BF16_KERNEL_SIGNATURES = {
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _I, _VP, _SZ, _VP],
+    "zk_moe_experts_grouped": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
 }
 
 

@@ -153,6 +153,25 @@ class _Source:
         return self._cache[key]
 
 
+    def vectors(self, names: Sequence[str]) -> Tensor:
+        """The named tensors as float32, stacked along their first axis (one name: that tensor)."""
+        if len(names) == 1:
+            return self.vector(names[0])
+        key = ("vs",) + tuple(_strip(n, self.prefixes) for n in names)
+        if key not in self._cache:
+            shapes = [tuple(self._shape(n)) for n in names]
+            if any(s[1:] != shapes[0][1:] for s in shapes):
+                raise ValueError(f"cannot stack {list(zip(names, shapes))}")
+            out = self.rt.empty((sum(s[0] for s in shapes),) + shapes[0][1:], F32)
+            row = 0
+            for n, s in zip(names, shapes):
+                self._fill(n, out.rows(row, row + s[0]), 0)
+                row += s[0]
+            self.bytes_on_device += out.nbytes
+            self._cache[key] = out
+        return self._cache[key]
+
+
 class CheckpointWeights(_Source):
     """Tensors of a checked model folder, copied and converted on the device."""
 
