@@ -209,9 +209,18 @@ def route(x, router_w, top, dt):
     return ids, np.take_along_axis(s, ids, axis=1)
 
 
-def moe(x, w, pre, mlp, dt):
+def route_margins(x, router_w, top, dt):
+    """Per token, the gap between the last chosen router logit and the first one left out
+    (infinite when every expert is chosen): how close the choice was."""
+    z = np.sort(x.astype(dt) @ router_w.astype(dt).T, axis=1)[:, ::-1]
+    return z[:, top - 1] - z[:, top] if z.shape[1] > top else np.full(len(x), np.inf)
+
+
+def moe(x, w, pre, mlp, dt, margins=None):
     """sum over a token's chosen experts of expert(weight * x), plus the shared expert of x."""
     ids, wts = route(x, w[pre + "router"], mlp["router"]["top"], dt)
+    if margins is not None:
+        margins.append(route_margins(x, w[pre + "router"], mlp["router"]["top"], dt))
     out = np.zeros_like(x, dtype=dt)
     for t in range(x.shape[0]):
         for e, s in zip(ids[t], wts[t]):
@@ -234,9 +243,10 @@ def layer_calls(cfg):
     return calls + [(i, False) for i in range(loop["stop"], n)]
 
 
-def forward(cfg, w, tokens, dt=np.float64, trace=None):
+def forward(cfg, w, tokens, dt=np.float64, trace=None, margins=None):
     """Logits [T, vocab] of one sequence from position 0.  ``trace``: a list that receives the
-    residual stream after every layer run."""
+    residual stream after every layer run; ``margins``: one that receives, per routed layer run,
+    how close each token's choice of experts was."""
     tokens = np.asarray(tokens)
     pos = np.arange(len(tokens))
     eps = cfg["norm"]["eps"]
@@ -256,7 +266,7 @@ def forward(cfg, w, tokens, dt=np.float64, trace=None):
         else:
             raise ValueError(L["type"])
         if L.get("mlp"):
-            y = y + moe(h, w, pre + "mlp.", L["mlp"], dt)
+            y = y + moe(h, w, pre + "mlp.", L["mlp"], dt, margins)
         x = x + y
         if trace is not None:
             trace.append(x.copy())
