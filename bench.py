@@ -453,6 +453,38 @@ def gemma2_like(width, heads, kv_heads, dim, ff, groups, vocab, window):
                 vocab_size=vocab, sliding_window=window, max_position_embeddings=8192)
 
 
+def pubunex_config(width, heads, kv_heads, dim, ff, groups, vocab, window):
+    """``groups`` times (delta rule, attention with biases and scaled frequencies, latent attention),
+    each with eight routed experts of a quarter of the feed-forward size, two a token, and a shared
+    layer of half of it: as many feed-forward weights at work for a token as the dense layer beside it."""
+    moe = {"kind": "moe", "expert": {"ff": ff // 4, "limit": 7.0}, "router": {"experts": 8, "top": 2},
+           "shared": {"ff": ff // 2, "limit": 7.0}}
+    layers = []
+    for _ in range(groups):
+        layers += [
+            {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "conv": 4}, "mlp": dict(moe)},
+            {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                            "rot": {"base": 10000.0, "dims": dim // 2,
+                                                    "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}},
+             "mlp": dict(moe)},
+            {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim // 2, "rot_dim": dim // 4, "vdim": dim // 2,
+                                                   "kv_rank": 2 * dim, "scale": (3 * dim // 4) ** -0.5,
+                                                   "rot": {"base": 10000.0, "dims": dim // 4}}, "mlp": dict(moe)}]
+    return {"architecture": "Pubunex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": layers}
+
+
+# what is timed, beside which relative, against which plain implementation it is checked first, and
+# the deviations of the random tensors that are not drawn like matrices or gains
+DESIGNS = {
+    "dafotar": dict(name="Dafotar", make=dafotar_config, plain="dafotar_plain", std_of={".hc": 0.3, ".temp": 0.5, "canon": 0.3},
+                    beside=("gemma2", "Gemma 2", gemma2_like)),
+    "pubunex": dict(name="Pubunex", make=pubunex_config, plain="pubunex_plain",
+                    std_of={".conv": 0.3, "A_log": 0.5, "dt_bias": 0.5, "mix.norm": 1.0, "dkv.norm": 1.0, ".sink": 1.0, ".b": 0.02,
+                            "router": 0.1},
+                    beside=("dafotar", "Dafotar", dafotar_config)),
+}
+
+
 def state_bytes_touched(model):
     """Bytes of per-request state a decoded token reads and writes (recurrences, convolutions)."""
     from zse_amd.parts.base import StateNeed
@@ -463,13 +495,14 @@ def state_bytes_touched(model):
     return total
 
 
-def check_design_slice(cfg, rt, seed, std, gain_std, std_of):
-    """The first three layers of the Dafotar model that is timed, at full width, against the plain
+def check_design_slice(cfg, rt, seed, std, gain_std, std_of, plain="dafotar_plain"):
+    """The first three layers of the model that is timed, at full width, against the plain
     implementation under ``tests/plain`` on the same weights made on the host: a prompt of 150 tokens
     whole (the mLSTM's chunks side by side), another in portions and then token by token beside a
     third, in 32-bit and in bfloat16.  The head is restricted to the first 4,096 rows of the embedding."""
+    import importlib
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from plain import dafotar_plain as P
+    P = importlib.import_module("plain." + plain)
     from zse_amd.engine.loading import random_model
     from zse_amd.engine.model import Model
     from zse_amd.engine.runner import StepEntry, StepRunner
@@ -515,22 +548,24 @@ def check_design_slice(cfg, rt, seed, std, gain_std, std_of):
 
 
 def run_design(a):
-    """Prefill and decode of Dafotar beside Gemma 2 at equal layer sizes; one JSON line."""
+    """Prefill and decode of a design beside its closest relative at equal layer sizes; one JSON line."""
     from zse_amd.engine.loading import random_model
     from zse_amd.runtime.device import Runtime
     rt = Runtime.get()
     sizes = [s for s in a.design_sizes.split(",") if s]
-    out = {"design": "Dafotar", "beside": "Gemma 2 at equal layer sizes", "dtype": "bf16", "data": "synthetic",
+    design = DESIGNS[a.design]
+    other, other_name, other_make = design["beside"]
+    out = {"design": design["name"], "beside": f"{other_name} at equal layer sizes", "dtype": "bf16", "data": "synthetic",
            "batch": a.batch, "context": a.context, "prefill_tokens": a.prefill_tokens, "sizes": {}}
     for name in sizes:
         size = DESIGN_SIZES[name]
         rec = {"config": size}
-        std_of = {".hc": 0.3, ".temp": 0.5, "canon": 0.3}
-        for which, cfg in (("dafotar", dafotar_config(**size)), ("gemma2", gemma2_like(**size))):
+        for which, cfg in ((a.design, design["make"](**size)), (other, other_make(**size))):
             if a.only_model and which != a.only_model:
                 continue
-            if which == "dafotar" and not a.no_check and not a.only:
-                errs = check_design_slice(cfg, rt, 0, 0.02, 0.1, std_of)
+            std_of = DESIGNS[which]["std_of"] if which in DESIGNS else {}
+            if which == a.design and not a.no_check and not a.only:
+                errs = check_design_slice(cfg, rt, 0, 0.02, 0.1, std_of, design["plain"])
                 rec["check"] = {"fp32_max_rel_err": float(f"{errs['float32']:.3g}"), "bf16_max_rel_err": float(f"{errs['bfloat16']:.3g}"),
                                 "slice_layers": 3, "cuts": "whole, portions, token by token, mixed"}
                 log(f"{name} check against the plain implementation: {rec['check']}")
@@ -565,10 +600,11 @@ def run_design(a):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["dafotar"], default=None,
-                    help="instead of the default workload: prefill and decode of this design beside Gemma 2 at equal layer sizes")
+    ap.add_argument("--design", choices=sorted(DESIGNS), default=None,
+                    help="instead of the default workload: prefill and decode of this design beside its closest relative "
+                         "(Dafotar beside Gemma 2, Pubunex beside Dafotar) at equal layer sizes")
     ap.add_argument("--design-sizes", default="w1024,w2048,w4096", help="with --design: which of " + ", ".join(DESIGN_SIZES))
-    ap.add_argument("--only-model", choices=["dafotar", "gemma2"], default=None, help="with --design, a profiling aid: one of the two")
+    ap.add_argument("--only-model", choices=["dafotar", "gemma2", "pubunex"], default=None, help="with --design, a profiling aid: one of the two")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)

@@ -305,6 +305,63 @@ def test_wide_latent_rows(dev):
     assert np.abs(rt.download(o).reshape(T, H, C) - want).max() < 2e-5
 
 
+@pytest.mark.parametrize("H,C,R,bs", [(3, 20, 4, 8), (16, 256, 32, 16), (5, 96, 16, 4), (40, 64, 8, 16)])
+def test_latent_attention_on_the_matrix_cores(H, C, R, bs):
+    """Three requests in one step: a long portion from position 0, a portion behind a context, and
+    one token behind a long context (its keys cut into ranges and joined); heads that do not fill
+    a tile of rows, rows of one token that spread over two tiles, and sinks."""
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(H)
+    HD = C + R
+    reqs = [(0, 150), (70, 37), (333, 1)]                          # (tokens already cached, tokens in the step)
+    T = sum(n for _, n in reqs)
+    sinks = rng.normal(0, 1, H).astype(np.float32)
+    scale = 2.0 / np.sqrt(HD)
+    max_ctx = max(a + n for a, n in reqs)
+    max_blocks = -(-max_ctx // bs)
+    pages = sum(-(-(a + n) // bs) for a, n in reqs)
+    cache = np.zeros((pages + 1, 1, bs, HD), np.float32)
+    table = np.full((len(reqs), max_blocks), -1, np.int32)
+    order = rng.permutation(pages) + 1
+    q_rows, want, q_start, ctx_len, positions, at = [], [], [0], [], [], 0
+    for r, (a, n) in enumerate(reqs):
+        L = a + n
+        rows = bf16(rng.normal(0, 1, (L, HD)))
+        mine = order[at:at + -(-L // bs)]
+        at += len(mine)
+        table[r, :len(mine)] = mine
+        for j in range(L):
+            cache[mine[j // bs], 0, j % bs] = rows[j]
+        q = bf16(rng.normal(0, 1, (L, H, HD)))
+        full = P.causal_attention(q.astype(np.float64), rows[:, None].astype(np.float64), rows[:, None, :C].astype(np.float64),
+                                  scale, sinks, np.float64)
+        q_rows.append(q[a:])
+        want.append(full[a:])
+        q_start.append(q_start[-1] + n)
+        ctx_len.append(L)
+        positions += list(range(a, L))
+    q_all, want = np.concatenate(q_rows), np.concatenate(want)
+    work = rt.empty((int(k.zk_latent_attention_bf16_workspace(32, H, C, 32)) // 4,), "float32")
+    out = rt.empty((T, H * C), "bfloat16")
+    d_cache = up16(rt, cache)
+    for with_work in (True, False):
+        k.zk_latent_attention_bf16(up16(rt, q_all).ptr, d_cache.ptr, up(rt, table).ptr, max_blocks, i32(rt, q_start).ptr,
+                                   i32(rt, ctx_len).ptr, i32(rt, positions).ptr, up(rt, sinks).ptr, out.ptr,
+                                   work.ptr if with_work else None, work.nbytes if with_work else 0, T, len(reqs), 160, 512, H,
+                                   HD, C, bs, scale, rt.stream)
+        got = rt.download_f32(out).reshape(T, H, C)
+        assert np.abs(got - want).max() < 0.03 * np.abs(want).max(), with_work
+    # the single token alone: few blocks, so its keys are cut into ranges
+    a, n = reqs[2]
+    k.zk_latent_attention_bf16(up16(rt, q_all[-1:]).ptr, d_cache.ptr, up(rt, table[2:]).ptr, max_blocks, i32(rt, [0, 1]).ptr,
+                               i32(rt, [a + n]).ptr, i32(rt, [a]).ptr, up(rt, sinks).ptr, out.ptr, work.ptr, work.nbytes, 1, 1, 1,
+                               512, H, HD, C, bs, scale, rt.stream)
+    got = rt.download_f32(out).reshape(T, H, C)[0]
+    assert np.abs(got - want[-1]).max() < 0.03 * np.abs(want).max()
+
+
 def test_biases_and_scaled_rotation_in_front_of_an_attention(dev):
     rt, k = dev
     rng = np.random.default_rng(11)

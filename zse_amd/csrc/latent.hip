@@ -152,3 +152,260 @@ int zk_heads_linear(const void* x, int ldx, int x_head, const void* w, int w_kn,
 
 ZK_ENTER(zk_latent_prep)
 ZK_ENTER(zk_heads_linear)
+
+#if ZSE_ACT_BF16
+// ---- the attention itself on the matrix cores (bfloat16)
+// Every head of a token reads the same cached rows, so the rows of the first product are
+// (token, head) pairs: row i of a request's step is head i % H of its token i / H.  A block takes
+// up to 128 such rows (a wave 32 of them) and walks the keys in tiles of 32 that all its waves
+// share through local memory, once as they lie (for S^T = K Q^T) and once transposed (their first
+// C channels are the values: O^T += V^T P^T).  Both products keep a row in a fixed lane (column =
+// lane % 32), so the running maximum and sum are per-lane numbers, and the weights a lane holds
+// after the first product are its operand of the second: the order of the keys in that product
+// is permuted to match (slots e < 4 of lane half h are keys 4h + e, slots e >= 4 keys 8 + 4h + e - 4).
+// Few rows behind long contexts: the keys are cut into ranges over blockIdx.z, every block
+// leaves (max, sum, O) of its range and a second kernel joins them; the sink enters there.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float floatx16_t __attribute__((ext_vector_type(16)));
+
+#define LA_ROWS 128
+#define LA_VT_LD 40
+
+template <int DT>
+__global__ __launch_bounds__(256) void latent_attn_kernel(
+    const __bf16* __restrict__ qa, const __bf16* __restrict__ kcache, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, const float* __restrict__ sinks,
+    __bf16* __restrict__ out, float* __restrict__ part, int H, int HD, int C, int HDP, int bs, float scale, int splits,
+    int split_keys) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int LDK = HDP + 8;
+  __bf16* Ks = (__bf16*)smem;                       // [32][LDK]
+  __bf16* Vt = Ks + 32 * LDK;                       // [DT * 32][LA_VT_LD]
+  __bf16* Qs = Vt + DT * 32 * LA_VT_LD;             // [LA_ROWS][LDK]
+  const int r = blockIdx.y, split = blockIdx.z;
+  const int t0 = q_start[r], n_q = q_start[r + 1] - t0;
+  if (n_q <= 0) return;
+  const int rows = n_q * H, row0 = blockIdx.x * LA_ROWS;
+  if (row0 >= rows) return;
+  const int ctx = ctx_len[r];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, lh = lane >> 5;
+  const int pieces = HDP / 8;
+  const int* table = block_table + (size_t)r * max_blocks;
+  for (int i = tid; i < LA_ROWS * pieces; i += 256) {
+    const int row = i / pieces, c8 = (i % pieces) * 8;
+    bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (row0 + row < rows && c8 < HD) v = *(const bf16x8_t*)(qa + ((size_t)t0 * H + row0 + row) * HD + c8);
+    *(bf16x8_t*)(Qs + row * LDK + c8) = v;
+  }
+  const int wrow = row0 + wave * 32 + lr;
+  const int my_pos = wrow < rows ? ctx - n_q + wrow / H : -1;
+  const bool wave_live = row0 + wave * 32 < rows;
+  const int last_row = min(rows, row0 + LA_ROWS) - 1;
+  const int k_begin = split * split_keys;
+  const int k_end = min(ctx - n_q + last_row / H + 1, (split + 1) * split_keys);      // exclusive
+  float m = -INFINITY, l = 0.f;
+  floatx16_t o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
+  for (int key0 = k_begin; key0 < k_end; key0 += 32) {
+    __syncthreads();                                 // the last tile has been used (and Q is in place)
+    for (int i = tid; i < 32 * pieces; i += 256) {
+      const int kk = i / pieces, c8 = (i % pieces) * 8, key = key0 + kk;
+      bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (key < k_end && c8 < HD) {
+        const int page = table[key / bs];
+        v = *(const bf16x8_t*)(kcache + ((size_t)page * bs + key % bs) * HD + c8);
+      }
+      *(bf16x8_t*)(Ks + kk * LDK + c8) = v;
+      if (c8 < DT * 32) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) Vt[(c8 + j) * LA_VT_LD + kk] = (c8 + j < C) ? v[j] : (__bf16)0.f;
+      }
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+    floatx16_t s;
+#pragma unroll
+    for (int e = 0; e < 16; e++) s[e] = 0.f;
+    const __bf16* ka = Ks + lr * LDK + lh * 8;
+    const __bf16* qb = Qs + (wave * 32 + lr) * LDK + lh * 8;
+    for (int ks = 0; ks < HDP / 16; ks++)
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(const bf16x8_t*)(ka + ks * 16), *(const bf16x8_t*)(qb + ks * 16), s, 0, 0, 0);
+    float mt = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const int key = key0 + (e / 4) * 8 + lh * 4 + (e % 4);
+      const bool seen = key <= my_pos && key < k_end;
+      s[e] = seen ? s[e] * scale : -INFINITY;
+      mt = fmaxf(mt, s[e]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float m_new = fmaxf(m, mt);
+    const float corr = (m_new == -INFINITY) ? 1.f : __expf(m - m_new);
+    float p[16], ps = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      p[e] = (s[e] == -INFINITY) ? 0.f : __expf(s[e] - m_new);
+      ps += p[e];
+    }
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * corr + ps;
+    m = m_new;
+    bf16x8_t pb0, pb1;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      pb0[e] = (__bf16)p[e];
+      pb1[e] = (__bf16)p[8 + e];
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[dt][e] *= corr;
+      const __bf16* vr = Vt + (dt * 32 + lr) * LA_VT_LD + 4 * lh;
+      const bf16x4_t a0 = *(const bf16x4_t*)vr, a1 = *(const bf16x4_t*)(vr + 8);
+      const bf16x4_t a2 = *(const bf16x4_t*)(vr + 16), a3 = *(const bf16x4_t*)(vr + 24);
+      bf16x8_t va, vb;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        va[e] = a0[e];
+        va[4 + e] = a1[e];
+        vb[e] = a2[e];
+        vb[4 + e] = a3[e];
+      }
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb0, o[dt], 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vb, pb1, o[dt], 0, 0, 0);
+    }
+  }
+  if (!wave_live || wrow >= rows) return;
+  const size_t grow = (size_t)t0 * H + wrow;          // the row's number in the step
+  if (splits > 1) {
+    const int CP = DT * 32;
+    float* pr = part + (grow * splits + split) * (size_t)(CP + 2);
+    if (lh == 0) {
+      pr[0] = m;
+      pr[1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) pr[2 + dt * 32 + (e / 4) * 8 + lh * 4 + (e % 4)] = o[dt][e];
+    return;
+  }
+  if (sinks != nullptr) {
+    const float sk = sinks[wrow % H];
+    const float m_new = fmaxf(m, sk);
+    const float corr = __expf(m - m_new);
+    l = l * corr + __expf(sk - m_new);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) o[dt][e] *= corr;
+  }
+  const float inv = 1.f / l;
+  __bf16* orow = out + grow * C;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const int d = dt * 32 + (e / 4) * 8 + lh * 4 + (e % 4);
+      if (d < C) orow[d] = (__bf16)(o[dt][e] * inv);
+    }
+}
+
+// One block per row of the step: joins the ranges' (max, sum, O), adds the sink.
+__global__ void latent_join_kernel(const float* __restrict__ part, const float* __restrict__ sinks,
+                                   const int* __restrict__ positions, __bf16* __restrict__ out, int H, int C, int CP,
+                                   int splits) {
+  const size_t row = blockIdx.x;
+  __bf16* orow = out + row * C;
+  if (positions[row / H] < 0) {                      // a padding row of a captured step
+    for (int c = threadIdx.x; c < C; c += blockDim.x) orow[c] = (__bf16)0.f;
+    return;
+  }
+  const float* pr = part + row * splits * (size_t)(CP + 2);
+  float M = sinks ? sinks[row % H] : -INFINITY;
+  for (int s = 0; s < splits; s++) M = fmaxf(M, pr[(size_t)s * (CP + 2)]);
+  float den = sinks ? __expf(sinks[row % H] - M) : 0.f;
+  for (int s = 0; s < splits; s++) {
+    const float ms = pr[(size_t)s * (CP + 2)];
+    if (ms > -INFINITY) den += pr[(size_t)s * (CP + 2) + 1] * __expf(ms - M);
+  }
+  const float inv = 1.f / den;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; s++) {
+      const float ms = pr[(size_t)s * (CP + 2)];
+      if (ms > -INFINITY) acc = fmaf(pr[(size_t)s * (CP + 2) + 2 + c], __expf(ms - M), acc);
+    }
+    orow[c] = (__bf16)(acc * inv);
+  }
+}
+
+extern "C" {
+
+// Whether the matrix-core kernel takes rows of HD channels of which the first C are values.
+int zk_latent_attention_bf16_supports(int HD, int C, int bs) {
+  return HD % 8 == 0 && HD <= 320 && C <= 256 && C <= HD && bs > 0;
+}
+
+// Floats of workspace that let a step of T tokens cut its keys into up to ``splits`` ranges.
+size_t zk_latent_attention_bf16_workspace(int T, int H, int C, int splits) {
+  const int CP = C <= 64 ? 64 : C <= 128 ? 128 : 256;
+  return (size_t)T * H * splits * (CP + 2) * sizeof(float);
+}
+
+// qa: [T, H, HD] queries carried over to the cached rows' channels; kcache: [pages, 1, bs, HD];
+// out: [T, H, C].  Request r holds rows [q_start[r], q_start[r + 1]) and ends at position
+// ctx_len[r] - 1.  max_q_len, max_ctx: the longest portion and context of the step (they size
+// the grid).  work: float scratch of work_bytes (may be null: no ranges).
+int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* block_table, int max_blocks,
+                             const int* q_start, const int* ctx_len, const int* positions, const float* sinks, void* out,
+                             void* work, size_t work_bytes, int T, int R, int max_q_len, int max_ctx, int H, int HD, int C,
+                             int bs, float scale, void* stream) {
+  ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && max_q_len > 0 && max_ctx > 0 && max_blocks > 0, "zk_latent_attention_bf16: bad sizes");
+  ZK_REQUIRE(zk_latent_attention_bf16_supports(HD, C, bs), "zk_latent_attention_bf16: rows of up to 320 channels in eights, up to 256 of them values");
+  ZK_REQUIRE(R <= 65535, "zk_latent_attention_bf16: too many requests");
+  if (T == 0 || R == 0) return 0;
+  const int HDP = (HD + 15) / 16 * 16;
+  const int DT = C <= 64 ? 2 : C <= 128 ? 4 : 8;
+  const int groups = (int)(((size_t)max_q_len * H + LA_ROWS - 1) / LA_ROWS);
+  int splits = 1;
+  const int blocks = groups * R;
+  if (blocks < 128 && work != nullptr) {
+    splits = (256 + blocks - 1) / blocks;
+    splits = min(splits, (max_ctx + 127) / 128);
+    splits = min(splits, 64);
+    while (splits > 1 && zk_latent_attention_bf16_workspace(T, H, C, splits) > work_bytes) splits--;
+    splits = max(splits, 1);
+  }
+  const int split_keys = splits == 1 ? 0x40000000 : ((max_ctx + splits - 1) / splits + 31) / 32 * 32;
+  const size_t lds = ((size_t)32 * (HDP + 8) + (size_t)DT * 32 * LA_VT_LD + (size_t)LA_ROWS * (HDP + 8)) * sizeof(__bf16);
+  dim3 grid(groups, R, splits);
+  hipStream_t st = (hipStream_t)stream;
+#define LA_LAUNCH(N)                                                                                                   \
+  do {                                                                                                                 \
+    static bool raised = false;                                                                                        \
+    if (!raised) {                                                                                                     \
+      hipFuncSetAttribute((const void*)latent_attn_kernel<N>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+      raised = true;                                                                                                   \
+    }                                                                                                                  \
+    latent_attn_kernel<N><<<grid, 256, lds, st>>>((const __bf16*)qa, (const __bf16*)kcache, block_table, max_blocks,   \
+                                                  q_start, ctx_len, sinks, (__bf16*)out, (float*)work, H, HD, C, HDP,  \
+                                                  bs, scale, splits, split_keys);                                      \
+  } while (0)
+  if (DT == 2) LA_LAUNCH(2);
+  else if (DT == 4) LA_LAUNCH(4);
+  else LA_LAUNCH(8);
+#undef LA_LAUNCH
+  if (splits > 1)
+    latent_join_kernel<<<T * H, 128, 0, st>>>((const float*)work, sinks, positions, (__bf16*)out, H, C, DT * 32, splits);
+  return zk_launch_status("zk_latent_attention_bf16");
+}
+
+}  // extern "C"
+
+ZK_ENTER(zk_latent_attention_bf16)
+#endif

@@ -15,7 +15,7 @@ from __future__ import annotations
 
 from typing import List
 
-from ..runtime.device import Tensor
+from ..runtime.device import BF16, Tensor
 from .base import ROLE_GAIN, PagedKV, Part, TensorReq, build_part, register_part
 from .ops import linear
 
@@ -64,6 +64,22 @@ class LatentAttention(Part):
     def flops_per_token(self) -> float:
         return super().flops_per_token()     # the per-head products are the matrices up_k and up_v, once a token
 
+    SPLIT_ROWS, SPLITS = 32, 32              # tokens and ranges of keys that the workspace is sized for
+
+    def _fast(self, kernels, dtype: str, page_size: int) -> bool:
+        """Whether the matrix-core attention kernel serves this layer."""
+        s = self.spec
+        return bool(dtype == BF16 and not s.window and kernels.has("zk_latent_attention_bf16") and
+                    kernels.zk_latent_attention_bf16_supports(s.latent_dim + s.rotary_dim, s.latent_dim, page_size))
+
+    def prepare(self, kernels, dtype, max_seqs, max_model_len, page_size, max_batch_tokens=0) -> int:
+        """Workspace that lets steps of few rows behind long contexts cut their keys into ranges."""
+        if not self._fast(kernels, dtype, page_size):
+            return 0
+        s = self.spec
+        return int(kernels.zk_latent_attention_bf16_workspace(max(int(max_seqs), self.SPLIT_ROWS), s.num_heads,
+                                                               s.latent_dim, self.SPLITS))
+
     def flops_per_key(self) -> float:
         s = self.spec
         return 2.0 * s.num_heads * (2 * s.latent_dim + s.rotary_dim)
@@ -84,10 +100,16 @@ class LatentAttention(Part):
         # the plain part of every query head, carried over to the latent's channels
         k.zk_heads_linear(qd.ptr, ld, D + R, self.w_uk.ptr, 1, qa.ptr, H * (C + R), C + R, T, H, D, C, ctx.stream)
         o = ctx.alloc((T, H * C))
-        k.zk_attention_plain_sink(qa.ptr, H * (C + R), cache.k.ptr, cache.k.ptr, g.block_table, g.max_blocks,
-                                  ctx.req_of_token, ctx.positions, o.ptr, T, H, 1, C + R, C, g.page_size, float(s.scale),
-                                  0.0, int(s.window) if s.window else 0, 0, None, 0,
-                                  self.sinks.ptr if self.sinks is not None else None, 1, ctx.stream)
+        sinks = self.sinks.ptr if self.sinks is not None else None
+        if ctx.tuned and self._fast(k, ctx.dtype, g.page_size):
+            k.zk_latent_attention_bf16(qa.ptr, cache.k.ptr, g.block_table, g.max_blocks, ctx.q_start, ctx.ctx_len,
+                                       ctx.positions, sinks, o.ptr, ctx.workspace.ptr, ctx.workspace.nbytes, T, ctx.R,
+                                       max(int(ctx.max_q_len), 1), int(ctx.max_ctx), H, C + R, C, g.page_size,
+                                       float(s.scale), ctx.stream)
+        else:
+            k.zk_attention_plain_sink(qa.ptr, H * (C + R), cache.k.ptr, cache.k.ptr, g.block_table, g.max_blocks,
+                                      ctx.req_of_token, ctx.positions, o.ptr, T, H, 1, C + R, C, g.page_size,
+                                      float(s.scale), 0.0, int(s.window) if s.window else 0, 0, None, 0, sinks, 1, ctx.stream)
         v = ctx.alloc((T, H * E))
         k.zk_heads_linear(o.ptr, H * C, C, self.w_uv.ptr, 0, v.ptr, H * E, E, T, H, C, E, ctx.stream)
         return linear(ctx, v, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)

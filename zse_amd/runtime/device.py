@@ -203,6 +203,7 @@ BF16_KERNEL_SIGNATURES = {
     "zk_qkv_rope_bf16": [_VP, _I, _VP, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "zk_attention_bf16": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I,
                           _F, _F, _I, _I, _VP, _SZ, _VP],
+    "zk_latent_attention_bf16": [_VP, _VP, _VP, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _I, _I, _I, _I, _I, _I, _I, _I, _F, _VP],
     "zk_moe_experts_grouped": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
 }
 
@@ -306,6 +307,12 @@ class KernelLibrary:
             self._dll.zk_head_pick_bf16_workspace.restype = C.c_size_t
             self._dll.zk_head_pick_bf16_workspace.argtypes = [_I, _I]
             self.zk_head_pick_bf16_workspace = self._dll.zk_head_pick_bf16_workspace
+            self._dll.zk_latent_attention_bf16_supports.restype = C.c_int
+            self._dll.zk_latent_attention_bf16_supports.argtypes = [_I, _I, _I]
+            self.zk_latent_attention_bf16_supports = self._dll.zk_latent_attention_bf16_supports
+            self._dll.zk_latent_attention_bf16_workspace.restype = C.c_size_t
+            self._dll.zk_latent_attention_bf16_workspace.argtypes = [_I, _I, _I, _I]
+            self.zk_latent_attention_bf16_workspace = self._dll.zk_latent_attention_bf16_workspace
             self._dll.zk_gemm_bf16_workspace.restype = C.c_size_t
             self._dll.zk_gemm_bf16_workspace.argtypes = []
             self.zk_gemm_bf16_workspace = self._dll.zk_gemm_bf16_workspace
