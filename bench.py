@@ -537,12 +537,23 @@ def check_design_slice(cfg, rt, seed, std, gain_std, std_of, plain="dafotar_plai
                 at += n
                 fed[e.req] += n
         assert all(fed[r] == len(t) for r, t in streams.items()), fed
-        worst = 0.0
+        worst, close = 0.0, 0
         for r, toks in streams.items():
-            want = P.forward(host_cfg, w, toks, np.float64)
+            # a design with routers: a token whose choice of experts is a close call in the plain run may
+            # go to another expert once the router's input is rounded to bfloat16; such rows are counted
+            # and left out of the bfloat16 bound (they stay in the 32-bit one)
+            margins = [] if "margins" in P.forward.__code__.co_varnames else None
+            want = P.forward(host_cfg, w, toks, np.float64, margins=margins) if margins is not None else \
+                P.forward(host_cfg, w, toks, np.float64)
             got = np.concatenate(rows[r]).astype(np.float64)
-            worst = max(worst, float(np.abs(got - want).max() / max(1e-9, np.abs(want).max())))
+            err = np.abs(got - want).max(axis=1) / max(1e-9, np.abs(want).max())
+            if dtype == "bfloat16" and margins:
+                calm = np.min(np.stack(margins), axis=0) > 0.08
+                close += int((~calm).sum())
+                err = err[calm]
+            worst = max(worst, float(err.max()) if err.size else 0.0)
         out[dtype] = worst
+        out["close_calls"] = close
         del runner, model
     return out
 
@@ -568,6 +579,8 @@ def run_design(a):
                 errs = check_design_slice(cfg, rt, 0, 0.02, 0.1, std_of, design["plain"])
                 rec["check"] = {"fp32_max_rel_err": float(f"{errs['float32']:.3g}"), "bf16_max_rel_err": float(f"{errs['bfloat16']:.3g}"),
                                 "slice_layers": 3, "cuts": "whole, portions, token by token, mixed"}
+                if errs.get("close_calls"):
+                    rec["check"]["rows_left_out_for_a_routers_close_call"] = errs["close_calls"]
                 log(f"{name} check against the plain implementation: {rec['check']}")
                 if not (errs["float32"] < 1e-4 and errs["bfloat16"] < 0.05):
                     raise SystemExit(f"bench.py: {name}: the engine does not agree with the plain implementation: {rec['check']}")

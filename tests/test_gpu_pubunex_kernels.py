@@ -89,7 +89,8 @@ def test_delta_rule_cut_into_steps(dev, H, G, D, E):
         k.zk_delta_rule(up(rt, qkv).ptr, ld, G * D, 2 * G * D, up(rt, z).ptr, H * E, up(rt, ba).ptr,
                         up(rt, A_log.astype(np.float32)).ptr, up(rt, dtb.astype(np.float32)).ptr,
                         up(rt, gain.astype(np.float32)).ptr, state.ptr, words, offset, i32(rt, q_start).ptr,
-                        i32(rt, [slot[0], slot[1]]).ptr, d_o.ptr, 2, H, G, D, E, eps, rt.stream)
+                        i32(rt, [slot[0], slot[1]]).ptr, i32(rt, list(range(T))).ptr, d_o.ptr,
+                        rt.empty((T, H * E), "float32").ptr, T, 2, H, G, D, E, eps, rt.stream)
         o = rt.download(d_o)
         for i, r in enumerate((0, 1)):
             got[r].append(o[q_start[i]:q_start[i + 1]])

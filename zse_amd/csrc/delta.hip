@@ -7,13 +7,16 @@
 // root mean square over E, times a gain [E] and silu(z_t).
 //
 // The recurrence never mixes value channels: column e of S, u and o depend on column e alone.
-// So a thread owns one column of S, D floats in registers, and walks the tokens of its request
-// without talking to any other thread; q_t and k_t are read from local memory by every thread
-// at the same address (a broadcast).  Tokens are staged in groups: the block loads and
-// normalises q and k of a group, walks it, then norms and gates the group's read-outs.  Every
-// sum runs in an order fixed by the channel numbers alone, so a request's values are the same
-// bits however its tokens are cut into steps.  All arithmetic is float; q, k, v, z come in the
-// activation type, b and a as floats.
+// Eight neighbouring lanes own one column of S, each a share of its rows in registers (row
+// chunks of four, dealt out in turn), and walk the tokens of their request; the two sums over
+// the rows (S^T k and S^T q) are joined across the eight lanes by three lane permutations inside
+// the wave, no local memory and no barrier.  q_t and k_t are read from local memory, every
+// column at the same addresses.  Tokens are staged in groups: the block loads and normalises q
+// and k of a group, walks it, then norms and gates the group's read-outs (a head whose value
+// channels span several blocks leaves that to a second kernel).  Every sum runs in an order
+// fixed by the channel numbers alone, so a request's values are the same bits however its
+// tokens are cut into steps.  All arithmetic is float; q, k, v, z come in the activation type,
+// b and a as floats.
 #include "common.h"
 #include "packed_call.h"
 
@@ -28,30 +31,49 @@ __device__ __forceinline__ float softplus_f(float x) {
   return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
 }
 
-template <int DMAX>
-__global__ void delta_rule_kernel(const act_t* __restrict__ qkv, int ld, int k_off, int v_off,
-                                  const act_t* __restrict__ z, int ldz, const float* __restrict__ ba,
-                                  const float* __restrict__ A_log, const float* __restrict__ dt_bias,
-                                  const float* __restrict__ gain, float* __restrict__ state, int slot_words,
-                                  int offset_words, const int* __restrict__ q_start,
-                                  const int* __restrict__ slot_of_req, act_t* __restrict__ out, int H, int G, int D,
-                                  int E, int Epad, float eps) {
-  extern __shared__ float lds[];
+#define DELTA_COLS 128            // value channels a block takes (8 lanes each: 1024 threads)
+
+// The sum of x over the 8 lanes that share a column: lane i with 7 - i, then inside the quads.
+__device__ __forceinline__ float sum8(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xf, 0xf, false));   // row_half_mirror
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false));    // quad_perm [1,0,3,2]
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false));    // quad_perm [2,3,0,1]
+  return x;
+}
+
+// RD: rows of S a lane holds (DMAX = 8 RD rows in all, D padded with zeros).  raw (may be null):
+// float [T, H * E], the read-outs before their norm, for a head that spans several blocks.
+template <int RD>
+__global__ __launch_bounds__(1024) void delta_rule_kernel(
+    const act_t* __restrict__ qkv, int ld, int k_off, int v_off, const act_t* __restrict__ z, int ldz,
+    const float* __restrict__ ba, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+    const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
+    const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
+    float* __restrict__ raw, int H, int G, int D, int E, float eps) {
+  constexpr int DMAX = 8 * RD, CH = RD / 4;          // CH: chunks of four rows a lane holds
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                 // [GROUP][DMAX]
   float* ks = qs + DELTA_GROUP * DMAX;             // [GROUP][DMAX]
-  float* ov = ks + DELTA_GROUP * DMAX;             // [GROUP][Epad]: v going in, the read-out coming back
-  float* beta = ov + DELTA_GROUP * Epad;           // [GROUP]
+  float* ov = ks + DELTA_GROUP * DMAX;             // [GROUP][DELTA_COLS]: v going in, the read-out coming back
+  float* beta = ov + DELTA_GROUP * DELTA_COLS;     // [GROUP]
   float* dec = beta + DELTA_GROUP;                 // [GROUP]
-  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
+  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * DELTA_COLS, tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+  const int col = tid >> 3, j = tid & 7, e = e0 + col;
   const int t0 = q_start[r], t1 = q_start[r + 1];
   if (t1 <= t0) return;
   const int g = h / (H / G);
-  const bool live = tid < E;
+  const bool live = e < E;
+  const int cols = min(DELTA_COLS, E - e0);
   float* S = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)h * D * E;
-  float s[DMAX];
+  float s[RD];
 #pragma unroll
-  for (int d = 0; d < DMAX; d++) s[d] = (live && d < D) ? S[(size_t)d * E + tid] : 0.f;
+  for (int i = 0; i < CH; i++)
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      const int d = 4 * (j + 8 * i) + c;
+      s[4 * i + c] = (live && d < D) ? S[(size_t)d * E + e] : 0.f;
+    }
   const float rate = expf(A_log[h]), shift = dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)D);
   for (int c0 = t0; c0 < t1; c0 += DELTA_GROUP) {
@@ -63,9 +85,9 @@ __global__ void delta_rule_kernel(const act_t* __restrict__ qkv, int ld, int k_o
       qs[i] = d < D ? to_f32(row[d]) : 0.f;
       ks[i] = d < D ? to_f32(row[k_off + d]) : 0.f;
     }
-    for (int i = tid; i < n * Epad; i += nt) {
-      const int tt = i / Epad, e = i % Epad;
-      ov[i] = e < E ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e]) : 0.f;
+    for (int i = tid; i < n * DELTA_COLS; i += nt) {
+      const int tt = i / DELTA_COLS, c = i % DELTA_COLS;
+      ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
     }
     if (tid < n) {
       const float* row = ba + (size_t)(c0 + tid) * 2 * H;
@@ -88,57 +110,95 @@ __global__ void delta_rule_kernel(const act_t* __restrict__ qkv, int ld, int k_o
       }
     }
     __syncthreads();
-    for (int tt = 0; tt < n; tt++) {               // the walk: nothing is shared between threads
-      const float4* k4 = (const float4*)(ks + tt * DMAX);
-      const float4* q4 = (const float4*)(qs + tt * DMAX);
+    for (int tt = 0; tt < n; tt++) {               // the walk: no barrier, three lane permutations a sum
+      const float4* k4 = (const float4*)(ks + tt * DMAX) + j;
+      const float4* q4 = (const float4*)(qs + tt * DMAX) + j;
       const float gt = dec[tt];
-      float dot = 0.f;
+      float4 kk[CH];
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
-      for (int d = 0; d < DMAX / 4; d++) {
-        const float4 kk = k4[d];
-        s[4 * d] *= gt;
-        s[4 * d + 1] *= gt;
-        s[4 * d + 2] *= gt;
-        s[4 * d + 3] *= gt;
-        dot = fmaf(s[4 * d], kk.x, dot);
-        dot = fmaf(s[4 * d + 1], kk.y, dot);
-        dot = fmaf(s[4 * d + 2], kk.z, dot);
-        dot = fmaf(s[4 * d + 3], kk.w, dot);
+      for (int i = 0; i < CH; i++) {
+        kk[i] = k4[8 * i];
+        s[4 * i] *= gt;
+        s[4 * i + 1] *= gt;
+        s[4 * i + 2] *= gt;
+        s[4 * i + 3] *= gt;
+        a0 = fmaf(s[4 * i], kk[i].x, a0);
+        a1 = fmaf(s[4 * i + 1], kk[i].y, a1);
+        a2 = fmaf(s[4 * i + 2], kk[i].z, a2);
+        a3 = fmaf(s[4 * i + 3], kk[i].w, a3);
       }
-      const float u = beta[tt] * (ov[tt * Epad + (live ? tid : 0)] - dot);
-      float o = 0.f;
+      const float dot = sum8((a0 + a1) + (a2 + a3));
+      const float u = beta[tt] * (ov[tt * DELTA_COLS + col] - dot);
+      a0 = a1 = a2 = a3 = 0.f;
 #pragma unroll
-      for (int d = 0; d < DMAX / 4; d++) {
-        const float4 kk = k4[d], qq = q4[d];
-        s[4 * d] = fmaf(kk.x, u, s[4 * d]);
-        s[4 * d + 1] = fmaf(kk.y, u, s[4 * d + 1]);
-        s[4 * d + 2] = fmaf(kk.z, u, s[4 * d + 2]);
-        s[4 * d + 3] = fmaf(kk.w, u, s[4 * d + 3]);
-        o = fmaf(s[4 * d], qq.x, o);
-        o = fmaf(s[4 * d + 1], qq.y, o);
-        o = fmaf(s[4 * d + 2], qq.z, o);
-        o = fmaf(s[4 * d + 3], qq.w, o);
+      for (int i = 0; i < CH; i++) {
+        const float4 qq = q4[8 * i];
+        s[4 * i] = fmaf(kk[i].x, u, s[4 * i]);
+        s[4 * i + 1] = fmaf(kk[i].y, u, s[4 * i + 1]);
+        s[4 * i + 2] = fmaf(kk[i].z, u, s[4 * i + 2]);
+        s[4 * i + 3] = fmaf(kk[i].w, u, s[4 * i + 3]);
+        a0 = fmaf(s[4 * i], qq.x, a0);
+        a1 = fmaf(s[4 * i + 1], qq.y, a1);
+        a2 = fmaf(s[4 * i + 2], qq.z, a2);
+        a3 = fmaf(s[4 * i + 3], qq.w, a3);
       }
-      if (live) ov[tt * Epad + tid] = o;
+      const float o = sum8((a0 + a1) + (a2 + a3));
+      // every lane of a column read v above before any of them writes the read-out here: the eight
+      // lanes of a column are in one wave and run in step
+      if (j == 0) ov[tt * DELTA_COLS + col] = o;
     }
     __syncthreads();
+    if (raw != nullptr) {                          // the head spans several blocks: its norm comes later
+      for (int i = tid; i < n * DELTA_COLS; i += nt) {
+        const int tt = i / DELTA_COLS, c = i % DELTA_COLS;
+        if (c < cols) raw[((size_t)(c0 + tt) * H + h) * E + e0 + c] = ov[i];
+      }
+      continue;
+    }
     for (int tt = wave; tt < n; tt += nw) {        // unit RMS over the head's read-out, gain, gate
       float ss = 0.f;
-      for (int e = lane; e < E; e += 64) ss = fmaf(ov[tt * Epad + e], ov[tt * Epad + e], ss);
+      for (int c = lane; c < E; c += 64) ss = fmaf(ov[tt * DELTA_COLS + c], ov[tt * DELTA_COLS + c], ss);
       ss = wave_sum(ss);
       const float inv = 1.0f / sqrtf(ss / (float)E + eps);
       const act_t* zr = z + (size_t)(c0 + tt) * ldz + (size_t)h * E;
       act_t* orow = out + ((size_t)(c0 + tt) * H + h) * E;
-      for (int e = lane; e < E; e += 64) {
-        const float zz = to_f32(zr[e]);
-        orow[e] = from_f32<act_t>(ov[tt * Epad + e] * inv * gain[e] * (zz / (1.0f + expf(-zz))));
+      for (int c = lane; c < E; c += 64) {
+        const float zz = to_f32(zr[c]);
+        orow[c] = from_f32<act_t>(ov[tt * DELTA_COLS + c] * inv * gain[c] * (zz / (1.0f + expf(-zz))));
       }
     }
   }
   if (live) {
 #pragma unroll
-    for (int d = 0; d < DMAX; d++)
-      if (d < D) S[(size_t)d * E + tid] = s[d];
+    for (int i = 0; i < CH; i++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int d = 4 * (j + 8 * i) + c;
+        if (d < D) S[(size_t)d * E + e] = s[4 * i + c];
+      }
+  }
+}
+
+// One wave per (token, head): out = raw / sqrt(mean(raw^2) + eps) * gain * silu(z).
+__global__ __launch_bounds__(64) void delta_finish_kernel(const float* __restrict__ raw, const act_t* __restrict__ z, int ldz,
+                                                          const float* __restrict__ gain, const int* __restrict__ positions,
+                                                          act_t* __restrict__ out, int H, int E, float eps) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* rr = raw + ((size_t)t * H + h) * E;
+  act_t* orow = out + ((size_t)t * H + h) * E;
+  if (positions[t] < 0) {                          // a padding row of a captured step
+    for (int c = lane; c < E; c += 64) orow[c] = from_f32<act_t>(0.f);
+    return;
+  }
+  float ss = 0.f;
+  for (int c = lane; c < E; c += 64) ss = fmaf(rr[c], rr[c], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)E + eps);
+  const act_t* zr = z + (size_t)t * ldz + (size_t)h * E;
+  for (int c = lane; c < E; c += 64) {
+    const float zz = to_f32(zr[c]);
+    orow[c] = from_f32<act_t>(rr[c] * inv * gain[c] * (zz / (1.0f + expf(-zz))));
   }
 }
 
@@ -148,37 +208,38 @@ extern "C" {
 // heads at k_off, H value heads of E at v_off.  z: [T, ldz], H heads of E (the output gate before
 // its silu).  ba: float [T, 2H], b then a.  A_log, dt_bias: float [H]; gain: float [E].
 // state: request r's S [H, D, E] lies at state[slot_of_req[r] * slot_words + offset_words].
-// out: [T, H * E].  Requests are rows [q_start[r], q_start[r + 1]).
+// out: [T, H * E].  Requests are rows [q_start[r], q_start[r + 1]).  raw: float scratch [T, H * E],
+// used by heads of more than 128 value channels (may be null for narrower ones); positions: [T].
 int zk_delta_rule(const void* qkv, int ld, int k_off, int v_off, const void* z, int ldz, const float* ba,
                   const float* A_log, const float* dt_bias, const float* gain, float* state, int slot_words,
-                  int offset_words, const int* q_start, const int* slot_of_req, void* out, int R, int H, int G, int D,
-                  int E, float eps, void* stream) {
-  ZK_REQUIRE(R >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && E > 0, "zk_delta_rule: bad sizes");
+                  int offset_words, const int* q_start, const int* slot_of_req, const int* positions, void* out,
+                  float* raw, int T, int R, int H, int G, int D, int E, float eps, void* stream) {
+  ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && E > 0, "zk_delta_rule: bad sizes");
   ZK_REQUIRE(D <= 256, "zk_delta_rule: up to 256 query/key channels a head");
-  ZK_REQUIRE(E <= 1024, "zk_delta_rule: up to 1024 value channels a head");
-  ZK_REQUIRE(H <= 65535, "zk_delta_rule: too many heads");
+  ZK_REQUIRE(H <= 65535 && (E + DELTA_COLS - 1) / DELTA_COLS <= 65535, "zk_delta_rule: too many heads or value channels");
   ZK_REQUIRE(state != nullptr && slot_words >= offset_words + H * D * E, "zk_delta_rule: the state does not fit its slot");
-  if (R == 0) return 0;
-  const int threads = (E + 63) / 64 * 64, Epad = threads;
-  const int DMAX = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
-  const size_t lds = ((size_t)DELTA_GROUP * (2 * DMAX + Epad) + 2 * DELTA_GROUP) * sizeof(float);
-  dim3 grid(R, H);
-#define LAUNCH(N)                                                                                                      \
-  do {                                                                                                                 \
-    static bool raised = false;                                                                                        \
-    if (lds > 48 * 1024 && !raised) {                                                                                  \
-      hipFuncSetAttribute((const void*)delta_rule_kernel<N>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-      raised = true;                                                                                                   \
-    }                                                                                                                  \
-    delta_rule_kernel<N><<<grid, threads, lds, (hipStream_t)stream>>>(                                                 \
-        (const act_t*)qkv, ld, k_off, v_off, (const act_t*)z, ldz, ba, A_log, dt_bias, gain, state, slot_words,        \
-        offset_words, q_start, slot_of_req, (act_t*)out, H, G, D, E, Epad, eps);                                       \
-  } while (0)
-  if (DMAX == 32) LAUNCH(32);
-  else if (DMAX == 64) LAUNCH(64);
-  else if (DMAX == 128) LAUNCH(128);
-  else LAUNCH(256);
+  const int blocks_e = (E + DELTA_COLS - 1) / DELTA_COLS;
+  ZK_REQUIRE(blocks_e == 1 || (raw != nullptr && positions != nullptr), "zk_delta_rule: heads of more than 128 value channels need scratch");
+  if (R == 0 || T == 0) return 0;
+  const int cols = E < DELTA_COLS ? (E + 7) / 8 * 8 : DELTA_COLS;       // whole waves: 8 columns each
+  const int threads = cols * 8;
+  const int RD = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
+  const size_t lds = ((size_t)DELTA_GROUP * (2 * 8 * RD + DELTA_COLS) + 2 * DELTA_GROUP) * sizeof(float);
+  dim3 grid(R, H, blocks_e);
+  float* raw_arg = blocks_e > 1 ? raw : nullptr;
+#define LAUNCH(N)                                                                                                     \
+  delta_rule_kernel<N><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
+      (const act_t*)qkv, ld, k_off, v_off, (const act_t*)z, ldz, ba, A_log, dt_bias, gain, state, slot_words,         \
+      offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, G, D, E, eps)
+  if (RD == 4) LAUNCH(4);
+  else if (RD == 8) LAUNCH(8);
+  else if (RD == 16) LAUNCH(16);
+  else LAUNCH(32);
 #undef LAUNCH
+  if (blocks_e > 1) {
+    dim3 fg(T, H);
+    delta_finish_kernel<<<fg, 64, 0, (hipStream_t)stream>>>(raw, (const act_t*)z, ldz, gain, positions, (act_t*)out, H, E, eps);
+  }
   return zk_launch_status("zk_delta_rule");
 }
 

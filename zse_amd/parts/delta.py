@@ -12,7 +12,7 @@ is carried as floats in the request's state slot:
 Value head h reads query/key head h // (heads / kv_heads).  q, k, v and the gate are one
 product; b and a a second, small one whose results stay float.  The convolution's last
 ``taps - 1`` inputs are part of the request's state, behind S.  One kernel walks the tokens of
-every (request, head): a thread owns a column of S, so steps of single tokens and portions of
+every (request, head): eight lanes own a column of S, so steps of single tokens and portions of
 prompts run the same arithmetic in the same order.
 """
 from __future__ import annotations
@@ -87,9 +87,11 @@ class DeltaRule(Part):
         qkv = self.conv.forward(ctx, qkvz, cache.state_offset + self.state_words() * 4, ld=ld)
         out = ctx.alloc((T, self.vv))
         z_ptr = qkvz.ptr + (2 * self.qk + self.vv) * (4 if ctx.dtype == F32 else 2)
+        raw = ctx.alloc((T, self.vv), F32) if E > 128 else None       # a head that spans several blocks norms afterwards
         k.zk_delta_rule(qkv.ptr, 2 * self.qk + self.vv, self.qk, 2 * self.qk, z_ptr, ld, ba.ptr, self.A_log.ptr,
                         self.dt_bias.ptr, self.gain.ptr, ctx.state.ptr, ctx.state.shape[1], cache.state_offset // 4,
-                        ctx.q_start, ctx.slot_of_req, out.ptr, ctx.R, H, G, D, E, float(s.eps), ctx.stream)
+                        ctx.q_start, ctx.slot_of_req, ctx.positions, out.ptr, raw.ptr if raw is not None else None, T,
+                        ctx.R, H, G, D, E, float(s.eps), ctx.stream)
         return linear(ctx, out, self.w_o, ctx.alloc((T, s.hidden_size)), last_of=self)
 
 
