@@ -47,7 +47,7 @@ def up16(rt, a):
     return up(rt, f32_to_bf16_bits(np.asarray(a, np.float32)))
 
 
-@pytest.mark.parametrize("H,G,D,E", [(4, 2, 16, 24), (1, 1, 100, 70), (2, 2, 32, 130), (3, 1, 8, 8)])
+@pytest.mark.parametrize("H,G,D,E", [(4, 2, 16, 24), (1, 1, 100, 70), (2, 2, 32, 130), (3, 1, 8, 8), (2, 1, 200, 40)])
 def test_delta_rule_cut_into_steps(dev, H, G, D, E):
     """Two requests whose rows come in portions of unequal sizes, single rows among them; the
     state in the slot carries S from step to step, and a slot's other words stay untouched."""
@@ -90,7 +90,8 @@ def test_delta_rule_cut_into_steps(dev, H, G, D, E):
                         up(rt, A_log.astype(np.float32)).ptr, up(rt, dtb.astype(np.float32)).ptr,
                         up(rt, gain.astype(np.float32)).ptr, state.ptr, words, offset, i32(rt, q_start).ptr,
                         i32(rt, [slot[0], slot[1]]).ptr, i32(rt, list(range(T))).ptr, d_o.ptr,
-                        rt.empty((T, H * E), "float32").ptr, T, 2, H, G, D, E, eps, rt.stream)
+                        rt.empty((T, H * E), "float32").ptr, T, 2, max(cuts[0][step], cuts[1][step]), H, G, D, E, eps,
+                        rt.stream)
         o = rt.download(d_o)
         for i, r in enumerate((0, 1)):
             got[r].append(o[q_start[i]:q_start[i + 1]])

@@ -31,7 +31,8 @@ __device__ __forceinline__ float softplus_f(float x) {
   return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
 }
 
-#define DELTA_COLS 128            // value channels a block takes (8 lanes each: 1024 threads)
+#define DELTA_COLS 128            // the most value channels a block takes (8 lanes each: 1024 threads)
+#define DELTA_COLS_LONG 32        // and what it takes when portions are long: more blocks, one wave a SIMD
 
 // The sum of x over the 8 lanes that share a column: lane i with 7 - i, then inside the quads.
 __device__ __forceinline__ float sum8(float x) {
@@ -49,22 +50,22 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
     const float* __restrict__ ba, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
     const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
-    float* __restrict__ raw, int H, int G, int D, int E, float eps) {
-  constexpr int DMAX = 8 * RD, CH = RD / 4;          // CH: chunks of four rows a lane holds
+    float* __restrict__ raw, int H, int G, int D, int E, float eps, int COLS) {
+  constexpr int DMAX = 8 * RD, CH = RD / 4;          // CH: chunks of four rows a lane holds; COLS: value channels of this block
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;                                 // [GROUP][DMAX]
   float* ks = qs + DELTA_GROUP * DMAX;             // [GROUP][DMAX]
-  float* ov = ks + DELTA_GROUP * DMAX;             // [GROUP][DELTA_COLS]: v going in, the read-out coming back
-  float* beta = ov + DELTA_GROUP * DELTA_COLS;     // [GROUP]
+  float* ov = ks + DELTA_GROUP * DMAX;             // [GROUP][COLS]: v going in, the read-out coming back
+  float* beta = ov + DELTA_GROUP * COLS;           // [GROUP]
   float* dec = beta + DELTA_GROUP;                 // [GROUP]
-  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * DELTA_COLS, tid = threadIdx.x, nt = blockDim.x;
+  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * COLS, tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
   const int col = tid >> 3, j = tid & 7, e = e0 + col;
   const int t0 = q_start[r], t1 = q_start[r + 1];
   if (t1 <= t0) return;
   const int g = h / (H / G);
   const bool live = e < E;
-  const int cols = min(DELTA_COLS, E - e0);
+  const int cols = min(COLS, E - e0);
   float* S = state + (size_t)slot_of_req[r] * slot_words + offset_words + (size_t)h * D * E;
   float s[RD];
 #pragma unroll
@@ -85,8 +86,8 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
       qs[i] = d < D ? to_f32(row[d]) : 0.f;
       ks[i] = d < D ? to_f32(row[k_off + d]) : 0.f;
     }
-    for (int i = tid; i < n * DELTA_COLS; i += nt) {
-      const int tt = i / DELTA_COLS, c = i % DELTA_COLS;
+    for (int i = tid; i < n * COLS; i += nt) {
+      const int tt = i / COLS, c = i % COLS;
       ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
     }
     if (tid < n) {
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
         a3 = fmaf(s[4 * i + 3], kk[i].w, a3);
       }
       const float dot = sum8((a0 + a1) + (a2 + a3));
-      const float u = beta[tt] * (ov[tt * DELTA_COLS + col] - dot);
+      const float u = beta[tt] * (ov[tt * COLS + col] - dot);
       a0 = a1 = a2 = a3 = 0.f;
 #pragma unroll
       for (int i = 0; i < CH; i++) {
@@ -146,26 +147,26 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
       const float o = sum8((a0 + a1) + (a2 + a3));
       // every lane of a column read v above before any of them writes the read-out here: the eight
       // lanes of a column are in one wave and run in step
-      if (j == 0) ov[tt * DELTA_COLS + col] = o;
+      if (j == 0) ov[tt * COLS + col] = o;
     }
     __syncthreads();
     if (raw != nullptr) {                          // the head spans several blocks: its norm comes later
-      for (int i = tid; i < n * DELTA_COLS; i += nt) {
-        const int tt = i / DELTA_COLS, c = i % DELTA_COLS;
+      for (int i = tid; i < n * COLS; i += nt) {
+        const int tt = i / COLS, c = i % COLS;
         if (c < cols) raw[((size_t)(c0 + tt) * H + h) * E + e0 + c] = ov[i];
       }
       continue;
     }
     for (int tt = wave; tt < n; tt += nw) {        // unit RMS over the head's read-out, gain, gate
       float ss = 0.f;
-      for (int c = lane; c < E; c += 64) ss = fmaf(ov[tt * DELTA_COLS + c], ov[tt * DELTA_COLS + c], ss);
+      for (int c = lane; c < E; c += 64) ss = fmaf(ov[tt * COLS + c], ov[tt * COLS + c], ss);
       ss = wave_sum(ss);
       const float inv = 1.0f / sqrtf(ss / (float)E + eps);
       const act_t* zr = z + (size_t)(c0 + tt) * ldz + (size_t)h * E;
       act_t* orow = out + ((size_t)(c0 + tt) * H + h) * E;
       for (int c = lane; c < E; c += 64) {
         const float zz = to_f32(zr[c]);
-        orow[c] = from_f32<act_t>(ov[tt * DELTA_COLS + c] * inv * gain[c] * (zz / (1.0f + expf(-zz))));
+        orow[c] = from_f32<act_t>(ov[tt * COLS + c] * inv * gain[c] * (zz / (1.0f + expf(-zz))));
       }
     }
   }
@@ -209,28 +210,32 @@ extern "C" {
 // its silu).  ba: float [T, 2H], b then a.  A_log, dt_bias: float [H]; gain: float [E].
 // state: request r's S [H, D, E] lies at state[slot_of_req[r] * slot_words + offset_words].
 // out: [T, H * E].  Requests are rows [q_start[r], q_start[r + 1]).  raw: float scratch [T, H * E],
-// used by heads of more than 128 value channels (may be null for narrower ones); positions: [T].
+// used by heads that span several blocks (may be null: a head of up to 128 value channels then stays
+// in one block whatever the step); positions: [T].  max_q_len: the longest portion of the step: with
+// long portions a block takes 32 value channels, so that a head's walk spreads over more compute units.
 int zk_delta_rule(const void* qkv, int ld, int k_off, int v_off, const void* z, int ldz, const float* ba,
                   const float* A_log, const float* dt_bias, const float* gain, float* state, int slot_words,
                   int offset_words, const int* q_start, const int* slot_of_req, const int* positions, void* out,
-                  float* raw, int T, int R, int H, int G, int D, int E, float eps, void* stream) {
+                  float* raw, int T, int R, int max_q_len, int H, int G, int D, int E, float eps, void* stream) {
   ZK_REQUIRE(T >= 0 && R >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && E > 0, "zk_delta_rule: bad sizes");
   ZK_REQUIRE(D <= 256, "zk_delta_rule: up to 256 query/key channels a head");
-  ZK_REQUIRE(H <= 65535 && (E + DELTA_COLS - 1) / DELTA_COLS <= 65535, "zk_delta_rule: too many heads or value channels");
+  ZK_REQUIRE(H <= 65535 && (E + DELTA_COLS_LONG - 1) / DELTA_COLS_LONG <= 65535, "zk_delta_rule: too many heads or value channels");
   ZK_REQUIRE(state != nullptr && slot_words >= offset_words + H * D * E, "zk_delta_rule: the state does not fit its slot");
-  const int blocks_e = (E + DELTA_COLS - 1) / DELTA_COLS;
-  ZK_REQUIRE(blocks_e == 1 || (raw != nullptr && positions != nullptr), "zk_delta_rule: heads of more than 128 value channels need scratch");
+  const bool scratch = raw != nullptr && positions != nullptr;
+  ZK_REQUIRE(E <= DELTA_COLS || scratch, "zk_delta_rule: heads of more than 128 value channels need scratch");
   if (R == 0 || T == 0) return 0;
-  const int cols = E < DELTA_COLS ? (E + 7) / 8 * 8 : DELTA_COLS;       // whole waves: 8 columns each
+  const int per_block = (scratch && max_q_len > DELTA_GROUP && E > DELTA_COLS_LONG) ? DELTA_COLS_LONG : DELTA_COLS;
+  const int blocks_e = (E + per_block - 1) / per_block;
+  const int cols = E < per_block ? (E + 7) / 8 * 8 : per_block;         // whole waves: 8 columns each
   const int threads = cols * 8;
   const int RD = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
-  const size_t lds = ((size_t)DELTA_GROUP * (2 * 8 * RD + DELTA_COLS) + 2 * DELTA_GROUP) * sizeof(float);
+  const size_t lds = ((size_t)DELTA_GROUP * (2 * 8 * RD + cols) + 2 * DELTA_GROUP) * sizeof(float);
   dim3 grid(R, H, blocks_e);
   float* raw_arg = blocks_e > 1 ? raw : nullptr;
 #define LAUNCH(N)                                                                                                     \
   delta_rule_kernel<N><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
       (const act_t*)qkv, ld, k_off, v_off, (const act_t*)z, ldz, ba, A_log, dt_bias, gain, state, slot_words,         \
-      offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, G, D, E, eps)
+      offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, G, D, E, eps, cols)
   if (RD == 4) LAUNCH(4);
   else if (RD == 8) LAUNCH(8);
   else if (RD == 16) LAUNCH(16);

@@ -192,7 +192,8 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lr = lane & 31, lh = lane >> 5;
   const int pieces = HDP / 8;
   const int* table = block_table + (size_t)r * max_blocks;
-  for (int i = tid; i < LA_ROWS * pieces; i += 256) {
+  const int staged = min(LA_ROWS, (rows - row0 + 31) / 32 * 32);      // the rows of waves that have any
+  for (int i = tid; i < staged * pieces; i += 256) {
     const int row = i / pieces, c8 = (i % pieces) * 8;
     bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
     if (row0 + row < rows && c8 < HD) v = *(const bf16x8_t*)(qa + ((size_t)t0 * H + row0 + row) * HD + c8);
@@ -210,22 +211,40 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   for (int dt = 0; dt < DT; dt++)
 #pragma unroll
     for (int e = 0; e < 16; e++) o[dt][e] = 0.f;
-  for (int key0 = k_begin; key0 < k_end; key0 += 32) {
-    __syncthreads();                                 // the last tile has been used (and Q is in place)
-    for (int i = tid; i < 32 * pieces; i += 256) {
+  // a tile's pieces travel from memory into registers while the tile before it is multiplied
+  constexpr int PRE = 5;                               // 16-byte pieces a thread carries: 32 x HDP / 8 / 256 <= 5 (HDP <= 320)
+  bf16x8_t nxt[PRE];
+  auto fetch = [&](int key0) {
+#pragma unroll
+    for (int u = 0; u < PRE; u++) {
+      const int i = tid + u * 256;
       const int kk = i / pieces, c8 = (i % pieces) * 8, key = key0 + kk;
       bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (key < k_end && c8 < HD) {
+      if (i < 32 * pieces && key < k_end && c8 < HD) {
         const int page = table[key / bs];
         v = *(const bf16x8_t*)(kcache + ((size_t)page * bs + key % bs) * HD + c8);
       }
-      *(bf16x8_t*)(Ks + kk * LDK + c8) = v;
-      if (c8 < DT * 32) {
+      nxt[u] = v;
+    }
+  };
+  if (k_begin < k_end) fetch(k_begin);
+  for (int key0 = k_begin; key0 < k_end; key0 += 32) {
+    __syncthreads();                                 // the last tile has been used (and Q is in place)
 #pragma unroll
-        for (int j = 0; j < 8; j++) Vt[(c8 + j) * LA_VT_LD + kk] = (c8 + j < C) ? v[j] : (__bf16)0.f;
+    for (int u = 0; u < PRE; u++) {
+      const int i = tid + u * 256;
+      if (i < 32 * pieces) {
+        const int kk = i / pieces, c8 = (i % pieces) * 8;
+        const bf16x8_t v = nxt[u];
+        *(bf16x8_t*)(Ks + kk * LDK + c8) = v;
+        if (c8 < DT * 32) {
+#pragma unroll
+          for (int j = 0; j < 8; j++) Vt[(c8 + j) * LA_VT_LD + kk] = (c8 + j < C) ? v[j] : (__bf16)0.f;
+        }
       }
     }
     __syncthreads();
+    if (key0 + 32 < k_end) fetch(key0 + 32);
     if (!wave_live) continue;
     floatx16_t s;
 #pragma unroll
@@ -316,9 +335,11 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
 }
 
 // One block per row of the step: joins the ranges' (max, sum, O), adds the sink.
-__global__ void latent_join_kernel(const float* __restrict__ part, const float* __restrict__ sinks,
-                                   const int* __restrict__ positions, __bf16* __restrict__ out, int H, int C, int CP,
-                                   int splits) {
+__global__ __launch_bounds__(256) void latent_join_kernel(const float* __restrict__ part, const float* __restrict__ sinks,
+                                                          const int* __restrict__ positions, __bf16* __restrict__ out, int H,
+                                                          int C, int CP, int splits) {
+  __shared__ float wgt[64];
+  __shared__ float inv_den;
   const size_t row = blockIdx.x;
   __bf16* orow = out + row * C;
   if (positions[row / H] < 0) {                      // a padding row of a captured step
@@ -326,21 +347,22 @@ __global__ void latent_join_kernel(const float* __restrict__ part, const float* 
     return;
   }
   const float* pr = part + row * splits * (size_t)(CP + 2);
-  float M = sinks ? sinks[row % H] : -INFINITY;
-  for (int s = 0; s < splits; s++) M = fmaxf(M, pr[(size_t)s * (CP + 2)]);
-  float den = sinks ? __expf(sinks[row % H] - M) : 0.f;
-  for (int s = 0; s < splits; s++) {
-    const float ms = pr[(size_t)s * (CP + 2)];
-    if (ms > -INFINITY) den += pr[(size_t)s * (CP + 2) + 1] * __expf(ms - M);
+  if (threadIdx.x < 64) {                            // one wave: the ranges' weights exp(m_s - M) and the denominator
+    const int s = threadIdx.x;
+    const float ms = s < splits ? pr[(size_t)s * (CP + 2)] : -INFINITY;
+    const float ls = s < splits ? pr[(size_t)s * (CP + 2) + 1] : 0.f;
+    const float sk = sinks ? sinks[row % H] : -INFINITY;
+    const float M = fmaxf(wave_max(ms), sk);
+    const float w = ms > -INFINITY ? __expf(ms - M) : 0.f;
+    const float den = wave_sum(ls * w) + (sinks ? __expf(sk - M) : 0.f);
+    wgt[s] = w;
+    if (s == 0) inv_den = 1.f / den;
   }
-  const float inv = 1.f / den;
+  __syncthreads();
   for (int c = threadIdx.x; c < C; c += blockDim.x) {
     float acc = 0.f;
-    for (int s = 0; s < splits; s++) {
-      const float ms = pr[(size_t)s * (CP + 2)];
-      if (ms > -INFINITY) acc = fmaf(pr[(size_t)s * (CP + 2) + 2 + c], __expf(ms - M), acc);
-    }
-    orow[c] = (__bf16)(acc * inv);
+    for (int s = 0; s < splits; s++) acc = fmaf(pr[(size_t)s * (CP + 2) + 2 + c], wgt[s], acc);
+    orow[c] = (__bf16)(acc * inv_den);
   }
 }
 
@@ -401,7 +423,7 @@ int zk_latent_attention_bf16(const void* qa, const void* kcache, const int* bloc
   else LA_LAUNCH(8);
 #undef LA_LAUNCH
   if (splits > 1)
-    latent_join_kernel<<<T * H, 128, 0, st>>>((const float*)work, sinks, positions, (__bf16*)out, H, C, DT * 32, splits);
+    latent_join_kernel<<<T * H, 256, 0, st>>>((const float*)work, sinks, positions, (__bf16*)out, H, C, DT * 32, splits);
   return zk_launch_status("zk_latent_attention_bf16");
 }
 

@@ -67,6 +67,35 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
   }
 }
 
+// Eight consecutive weights as floats (rows in whole groups of eight are read 16 bytes a lane).
+__device__ __forceinline__ void load8(const float* p, float v[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const __bf16* p, float v[8]) {
+  typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+  const b8 t = *(const b8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = (float)t[i];
+}
+
+// The dot product of a weight row and a row in local memory, over a wave; the same order of sums
+// whatever the step (eight channels a lane in turn where rows are whole groups of eight).
+__device__ __forceinline__ float row_dot(const act_t* __restrict__ w, const float* __restrict__ x, int n, int lane) {
+  float a = 0.f;
+  if ((n & 7) == 0) {
+    for (int i = lane * 8; i < n; i += 512) {
+      float v[8];
+      load8(w + i, v);
+#pragma unroll
+      for (int c = 0; c < 8; c++) a = fmaf(v[c], x[i + c], a);
+    }
+  } else {
+    for (int i = lane; i < n; i += 64) a = fmaf(to_f32(w[i]), x[i], a);
+  }
+  return wave_sum(a);
+}
+
 // ---- few tokens: y[(t, k), n] = act(Wg[e] x', Wu[e] x'), a wave per row pair
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(const act_t* __restrict__ x, const int* __restrict__ ids,
                                                           const float* __restrict__ wts, const act_t* __restrict__ w_gu,
@@ -85,13 +114,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const act_t* __restric
   for (int n = n0 + wave; n < min(F, n0 + rows_per_block); n += 4) {
     const act_t* gr = wg + (size_t)n * W;
     const act_t* ur = wg + (size_t)(F + n) * W;
-    float g = 0.f, u = 0.f;
-    for (int i = lane; i < W; i += 64) {
-      g = fmaf(to_f32(gr[i]), xs[i], g);
-      u = fmaf(to_f32(ur[i]), xs[i], u);
-    }
-    g = wave_sum(g);
-    u = wave_sum(u);
+    const float g = row_dot(gr, xs, W, lane), u = row_dot(ur, xs, W, lane);
     if (lane == 0) y[(size_t)pair * F + n] = from_f32<act_t>(clamped_swiglu(g, u, limit));
   }
 }
@@ -109,9 +132,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const act_t* __restrict__
     float total = 0.f;
     for (int k = 0; k < top; k++) {
       const act_t* wr = w_down + ((size_t)ids[(size_t)t * top + k] * W + n) * F;
-      float a = 0.f;
-      for (int i = lane; i < F; i += 64) a = fmaf(to_f32(wr[i]), ys[k * F + i], a);
-      total += wave_sum(a);
+      total += row_dot(wr, ys + k * F, F, lane);
     }
     if (lane == 0) out[(size_t)t * W + n] = total;
   }

@@ -62,7 +62,7 @@ int zk_attention_bf16(const void* q, int q_stride, const void* kcache, const voi
 
 namespace {
 
-constexpr int MOST_ARGS = 24;
+constexpr int MOST_ARGS = 32;
 
 // One written-down call: a row of the table, and the entry point's arguments as 64-bit words
 // in the order of its C signature.  The last argument of every entry point is the stream; a

@@ -184,7 +184,7 @@ KERNEL_SIGNATURES = {
     "zk_attention_plain_sink": [_VP, _I, _VP, _VP, _VP, _I, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _F,
                                 _I, _I, _VP, _I, _VP, _I, _VP],
     "zk_delta_rule": [_VP, _I, _I, _I, _VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I,
-                      _I, _F, _VP],
+                      _I, _I, _F, _VP],
     "zk_moe_route": [_VP, _VP, _VP, _I, _I, _I, _VP],
     "zk_moe_experts": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _F, _VP],
     "zk_clamped_glu": [_VP, _VP, _I, _I, _F, _VP],
