@@ -111,15 +111,38 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
       }
     }
     __syncthreads();
-    for (int tt = 0; tt < n; tt++) {               // the walk: no barrier, three lane permutations a sum
-      const float4* k4 = (const float4*)(ks + tt * DMAX) + j;
+    // the walk: no barrier, three lane permutations a sum.  What the next token needs first (its k, v,
+    // beta and decay) is asked for before this token's arithmetic, its q at the token's start.
+    float4 kn[CH];
+    float vn, bn, gn;
+    {
+      const float4* k4 = (const float4*)ks + j;
+#pragma unroll
+      for (int i = 0; i < CH; i++) kn[i] = k4[8 * i];
+      vn = ov[col];
+      bn = beta[0];
+      gn = dec[0];
+    }
+    for (int tt = 0; tt < n; tt++) {
       const float4* q4 = (const float4*)(qs + tt * DMAX) + j;
-      const float gt = dec[tt];
-      float4 kk[CH];
+      const float gt = gn, bt = bn, vt = vn;
+      float4 kk[CH], qq[CH];
+#pragma unroll
+      for (int i = 0; i < CH; i++) {
+        kk[i] = kn[i];
+        qq[i] = q4[8 * i];
+      }
+      if (tt + 1 < n) {
+        const float4* k4 = (const float4*)(ks + (tt + 1) * DMAX) + j;
+#pragma unroll
+        for (int i = 0; i < CH; i++) kn[i] = k4[8 * i];
+        vn = ov[(tt + 1) * COLS + col];
+        bn = beta[tt + 1];
+        gn = dec[tt + 1];
+      }
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
       for (int i = 0; i < CH; i++) {
-        kk[i] = k4[8 * i];
         s[4 * i] *= gt;
         s[4 * i + 1] *= gt;
         s[4 * i + 2] *= gt;
@@ -130,23 +153,22 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
         a3 = fmaf(s[4 * i + 3], kk[i].w, a3);
       }
       const float dot = sum8((a0 + a1) + (a2 + a3));
-      const float u = beta[tt] * (ov[tt * COLS + col] - dot);
+      const float u = bt * (vt - dot);
       a0 = a1 = a2 = a3 = 0.f;
 #pragma unroll
       for (int i = 0; i < CH; i++) {
-        const float4 qq = q4[8 * i];
         s[4 * i] = fmaf(kk[i].x, u, s[4 * i]);
         s[4 * i + 1] = fmaf(kk[i].y, u, s[4 * i + 1]);
         s[4 * i + 2] = fmaf(kk[i].z, u, s[4 * i + 2]);
         s[4 * i + 3] = fmaf(kk[i].w, u, s[4 * i + 3]);
-        a0 = fmaf(s[4 * i], qq.x, a0);
-        a1 = fmaf(s[4 * i + 1], qq.y, a1);
-        a2 = fmaf(s[4 * i + 2], qq.z, a2);
-        a3 = fmaf(s[4 * i + 3], qq.w, a3);
+        a0 = fmaf(s[4 * i], qq[i].x, a0);
+        a1 = fmaf(s[4 * i + 1], qq[i].y, a1);
+        a2 = fmaf(s[4 * i + 2], qq[i].z, a2);
+        a3 = fmaf(s[4 * i + 3], qq[i].w, a3);
       }
       const float o = sum8((a0 + a1) + (a2 + a3));
-      // every lane of a column read v above before any of them writes the read-out here: the eight
-      // lanes of a column are in one wave and run in step
+      // a column's v of this token was read (by its eight lanes, all in one wave) before the
+      // read-out takes its place
       if (j == 0) ov[tt * COLS + col] = o;
     }
     __syncthreads();

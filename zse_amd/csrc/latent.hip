@@ -114,6 +114,30 @@ __global__ __launch_bounds__(256) void heads_linear_kernel(const act_t* __restri
   }
 }
 
+// The same for steps of few tokens: a thread per column n, a block per (token, head, 64 columns);
+// the sum over k runs in the same order as in the tiled kernel, so a row's values are the same
+// bits whichever of the two computes it.
+template <bool KN>
+__global__ __launch_bounds__(64) void heads_linear_few_kernel(const act_t* __restrict__ x, int ldx, int x_head,
+                                                              const act_t* __restrict__ w, act_t* __restrict__ out, int ldo,
+                                                              int o_head, int K, int N) {
+  extern __shared__ float xrow[];                    // [K]
+  const int t = blockIdx.x, h = blockIdx.y, n = blockIdx.z * 64 + threadIdx.x;
+  const act_t* xr = x + (size_t)t * ldx + (size_t)h * x_head;
+  for (int k = threadIdx.x; k < K; k += 64) xrow[k] = to_f32(xr[k]);
+  __syncthreads();
+  if (n >= N) return;
+  const act_t* wh = w + (size_t)h * K * N;
+  float acc = 0.f;
+  if (KN) {
+    for (int k = 0; k < K; k++) acc = fmaf(xrow[k], to_f32(wh[(size_t)k * N + n]), acc);
+  } else {
+    const act_t* wr = wh + (size_t)n * K;
+    for (int k = 0; k < K; k++) acc = fmaf(xrow[k], to_f32(wr[k]), acc);
+  }
+  out[(size_t)t * ldo + (size_t)h * o_head + n] = from_f32<act_t>(acc);
+}
+
 extern "C" {
 
 // qd: [T, ld]: H query heads of D + R, then C + R of the down-projection.  qa: [T, H, C + R], of
@@ -138,6 +162,16 @@ int zk_heads_linear(const void* x, int ldx, int x_head, const void* w, int w_kn,
   ZK_REQUIRE(T >= 0 && H > 0 && K > 0 && N > 0, "zk_heads_linear: bad sizes");
   ZK_REQUIRE(H <= 65535 && (N + 63) / 64 <= 65535, "zk_heads_linear: too many heads or columns");
   if (T == 0) return 0;
+  if (T <= 16 && K <= 8192) {
+    dim3 few(T, H, (N + 63) / 64);
+    if (w_kn)
+      heads_linear_few_kernel<true><<<few, 64, (size_t)K * 4, (hipStream_t)stream>>>((const act_t*)x, ldx, x_head, (const act_t*)w,
+                                                                                    (act_t*)out, ldo, o_head, K, N);
+    else
+      heads_linear_few_kernel<false><<<few, 64, (size_t)K * 4, (hipStream_t)stream>>>((const act_t*)x, ldx, x_head, (const act_t*)w,
+                                                                                     (act_t*)out, ldo, o_head, K, N);
+    return zk_launch_status("zk_heads_linear");
+  }
   dim3 grid((T + HL_TT - 1) / HL_TT, H, (N + 63) / 64);
   if (w_kn)
     heads_linear_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>((const act_t*)x, ldx, x_head, (const act_t*)w,
@@ -217,8 +251,10 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
   auto fetch = [&](int key0) {
 #pragma unroll
     for (int u = 0; u < PRE; u++) {
+      // consecutive threads take consecutive keys of one column of pieces: the transposed copy is
+      // then written to consecutive addresses
       const int i = tid + u * 256;
-      const int kk = i / pieces, c8 = (i % pieces) * 8, key = key0 + kk;
+      const int kk = i & 31, c8 = (i >> 5) * 8, key = key0 + kk;
       bf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (i < 32 * pieces && key < k_end && c8 < HD) {
         const int page = table[key / bs];
@@ -234,7 +270,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(
     for (int u = 0; u < PRE; u++) {
       const int i = tid + u * 256;
       if (i < 32 * pieces) {
-        const int kk = i / pieces, c8 = (i % pieces) * 8;
+        const int kk = i & 31, c8 = (i >> 5) * 8;
         const bf16x8_t v = nxt[u];
         *(bf16x8_t*)(Ks + kk * LDK + c8) = v;
         if (c8 < DT * 32) {

@@ -65,7 +65,7 @@ int zk_sum_norm(float* h, const void* a, int a_parts, const void* b, int b_parts
   if (T == 0) return 0;
   // in the 32-bit library the block is always 256 wide: the order of a row's sums must not follow
   // from how many rows a step brings
-  const int threads = (ZSE_ACT_BF16 && T <= 64 && W >= 2048) ? 1024 : 256;
+  const int threads = (ZSE_ACT_BF16 && T <= 64 && W >= 1024) ? 1024 : 256;
   sum_norm_kernel<<<T, threads, 0, (hipStream_t)stream>>>(h, a, a_parts, b, b_parts, bias, w_next, eps, unit_offset,
                                                          (act_t*)out, W);
   return zk_launch_status("zk_sum_norm");
