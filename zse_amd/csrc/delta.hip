@@ -31,8 +31,26 @@ __device__ __forceinline__ float softplus_f(float x) {
   return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
 }
 
+// Eight consecutive activations as they lie in memory (16 bytes of bfloat16, or 32 of float, a
+// lane), turned into floats only when they are put down in local memory.
+#if ZSE_ACT_BF16
+typedef __bf16 Eight __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ Eight load8(const __bf16* p) { return *(const Eight*)p; }
+__device__ __forceinline__ float at8(const Eight& e, int i) { return (float)e[i]; }
+#else
+struct Eight {
+  float4 a, b;
+};
+__device__ __forceinline__ Eight load8(const float* p) { return Eight{*(const float4*)p, *(const float4*)(p + 4)}; }
+__device__ __forceinline__ float at8(const Eight& e, int i) {
+  const float4 h = i < 4 ? e.a : e.b;
+  const int c = i & 3;
+  return c == 0 ? h.x : c == 1 ? h.y : c == 2 ? h.z : h.w;
+}
+#endif
+
 #define DELTA_COLS 128            // the most value channels a block takes (8 lanes each: 1024 threads)
-#define DELTA_COLS_LONG 32        // and what it takes when portions are long: more blocks, one wave a SIMD
+#define DELTA_COLS_LONG 16        // and what it takes when portions are long: 16 lanes a column, more blocks, one wave a SIMD
 
 // The sum of x over the 8 lanes that share a column: lane i with 7 - i, then inside the quads.
 __device__ __forceinline__ float sum8(float x) {
@@ -42,25 +60,34 @@ __device__ __forceinline__ float sum8(float x) {
   return x;
 }
 
-// RD: rows of S a lane holds (DMAX = 8 RD rows in all, D padded with zeros).  raw (may be null):
-// float [T, H * E], the read-outs before their norm, for a head that spans several blocks.
-template <int RD>
-__global__ __launch_bounds__(1024) void delta_rule_kernel(
+// The sum over the 16 lanes of a row that share a column: lane i with 15 - i first.
+__device__ __forceinline__ float sum16(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xf, 0xf, false));   // row_mirror
+  return sum8(x);
+}
+
+// DS lanes share a column (8 or 16), each holds CH chunks of four rows of S (4 CH DS rows in all,
+// D padded with zeros).  raw (may be null): float [T, H * E], the read-outs before their norm,
+// for a head that spans several blocks.  GRP: tokens staged at a time.  PRE: pieces of eight q/k
+// values a thread carries for the next group of tokens (4: blocks of up to 256 threads, for long
+// portions; 1: blocks of up to 1024).
+template <int CH, int DS, int PRE>
+__global__ __launch_bounds__(PRE > 1 ? 256 : 1024) void delta_rule_kernel(
     const act_t* __restrict__ qkv, int ld, int k_off, int v_off, const act_t* __restrict__ z, int ldz,
     const float* __restrict__ ba, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
     const float* __restrict__ gain, float* __restrict__ state, int slot_words, int offset_words,
     const int* __restrict__ q_start, const int* __restrict__ slot_of_req, act_t* __restrict__ out,
-    float* __restrict__ raw, int H, int G, int D, int E, float eps, int COLS) {
-  constexpr int DMAX = 8 * RD, CH = RD / 4;          // CH: chunks of four rows a lane holds; COLS: value channels of this block
+    float* __restrict__ raw, int H, int G, int D, int E, float eps, int COLS, int GRP, int wide) {
+  constexpr int DMAX = 4 * CH * DS, RD = 4 * CH;     // RD: rows of S a lane holds; COLS: value channels of this block
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  float* qs = lds;                                 // [GROUP][DMAX]
-  float* ks = qs + DELTA_GROUP * DMAX;             // [GROUP][DMAX]
-  float* ov = ks + DELTA_GROUP * DMAX;             // [GROUP][COLS]: v going in, the read-out coming back
-  float* beta = ov + DELTA_GROUP * COLS;           // [GROUP]
-  float* dec = beta + DELTA_GROUP;                 // [GROUP]
+  float* qs = lds;                                 // [GRP][DMAX]
+  float* ks = qs + GRP * DMAX;                     // [GRP][DMAX]
+  float* ov = ks + GRP * DMAX;                     // [GRP][COLS]: v going in, the read-out coming back
+  float* beta = ov + GRP * COLS;                   // [GRP]
+  float* dec = beta + GRP;                         // [GRP]
   const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * COLS, tid = threadIdx.x, nt = blockDim.x;
   const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
-  const int col = tid >> 3, j = tid & 7, e = e0 + col;
+  const int col = tid / DS, j = tid % DS, e = e0 + col;
   const int t0 = q_start[r], t1 = q_start[r + 1];
   if (t1 <= t0) return;
   const int g = h / (H / G);
@@ -72,43 +99,95 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
   for (int i = 0; i < CH; i++)
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-      const int d = 4 * (j + 8 * i) + c;
+      const int d = 4 * (j + DS * i) + c;
       s[4 * i + c] = (live && d < D) ? S[(size_t)d * E + e] : 0.f;
     }
   const float rate = expf(A_log[h]), shift = dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)D);
-  for (int c0 = t0; c0 < t1; c0 += DELTA_GROUP) {
-    const int n = min(DELTA_GROUP, t1 - c0);
-    __syncthreads();
-    for (int i = tid; i < n * DMAX; i += nt) {
-      const int tt = i / DMAX, d = i % DMAX;
-      const act_t* row = qkv + (size_t)(c0 + tt) * ld + (size_t)g * D;
-      qs[i] = d < D ? to_f32(row[d]) : 0.f;
-      ks[i] = d < D ? to_f32(row[k_off + d]) : 0.f;
+  // wide: rows in whole groups of eight values.  A group's q, k, v, b and a are then asked for, 16
+  // bytes a lane, while the group before it is walked, and land in local memory afterwards.
+  const int qk_pieces = D / 8;                       // of one row of q (or k)
+  Eight pq[PRE], pv;
+  float pb = 0.f, pa = 0.f;
+  auto fetch = [&](int c0, int n) {
+#pragma unroll
+    for (int u = 0; u < PRE; u++) {
+      const int i = tid + u * nt;
+      if (i < 2 * n * qk_pieces) {
+        const int which = i / (n * qk_pieces), rest = i % (n * qk_pieces);
+        const int tt = rest / qk_pieces, d8 = (rest % qk_pieces) * 8;
+        pq[u] = load8(qkv + (size_t)(c0 + tt) * ld + (size_t)g * D + (which ? k_off : 0) + d8);
+      }
     }
-    for (int i = tid; i < n * COLS; i += nt) {
-      const int tt = i / COLS, c = i % COLS;
-      ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
+    if (tid < n * (COLS / 8)) {
+      const int tt = tid / (COLS / 8), c8 = (tid % (COLS / 8)) * 8;
+      if (c8 < cols) pv = load8(qkv + (size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c8);
     }
     if (tid < n) {
       const float* row = ba + (size_t)(c0 + tid) * 2 * H;
-      beta[tid] = 1.0f / (1.0f + expf(-row[h]));
-      dec[tid] = expf(-rate * softplus_f(row[H + h] + shift));
+      pb = row[h];
+      pa = row[H + h];
+    }
+  };
+  if (wide) {
+    for (int i = tid; i < GRP * DMAX; i += nt) qs[i] = ks[i] = 0.f;       // the rows' padding stays zero
+    for (int i = tid; i < GRP * COLS; i += nt) ov[i] = 0.f;
+    fetch(t0, min(GRP, t1 - t0));
+  }
+  for (int c0 = t0; c0 < t1; c0 += GRP) {
+    const int n = min(GRP, t1 - c0);
+    __syncthreads();
+    if (wide) {
+#pragma unroll
+      for (int u = 0; u < PRE; u++) {
+        const int i = tid + u * nt;
+        if (i < 2 * n * qk_pieces) {
+          const int which = i / (n * qk_pieces), rest = i % (n * qk_pieces);
+          const int tt = rest / qk_pieces, d8 = (rest % qk_pieces) * 8;
+          float* dst = (which ? ks : qs) + tt * DMAX + d8;
+#pragma unroll
+          for (int c = 0; c < 8; c++) dst[c] = at8(pq[u], c);
+        }
+      }
+      if (tid < n * (COLS / 8)) {
+        const int tt = tid / (COLS / 8), c8 = (tid % (COLS / 8)) * 8;
+        if (c8 < cols) {
+#pragma unroll
+          for (int c = 0; c < 8; c++) ov[tt * COLS + c8 + c] = at8(pv, c);
+        }
+      }
+      if (tid < n) {
+        beta[tid] = 1.0f / (1.0f + expf(-pb));
+        dec[tid] = expf(-rate * softplus_f(pa + shift));
+      }
+    } else {
+      for (int i = tid; i < n * DMAX; i += nt) {
+        const int tt = i / DMAX, d = i % DMAX;
+        const act_t* row = qkv + (size_t)(c0 + tt) * ld + (size_t)g * D;
+        qs[i] = d < D ? to_f32(row[d]) : 0.f;
+        ks[i] = d < D ? to_f32(row[k_off + d]) : 0.f;
+      }
+      for (int i = tid; i < n * COLS; i += nt) {
+        const int tt = i / COLS, c = i % COLS;
+        ov[i] = c < cols ? to_f32(qkv[(size_t)(c0 + tt) * ld + v_off + (size_t)h * E + e0 + c]) : 0.f;
+      }
+      if (tid < n) {
+        const float* row = ba + (size_t)(c0 + tid) * 2 * H;
+        beta[tid] = 1.0f / (1.0f + expf(-row[h]));
+        dec[tid] = expf(-rate * softplus_f(row[H + h] + shift));
+      }
     }
     __syncthreads();
-    for (int tt = wave; tt < n; tt += nw) {        // unit vectors
-      float sq = 0.f, sk = 0.f;
-      for (int d = lane; d < DMAX; d += 64) {
-        sq = fmaf(qs[tt * DMAX + d], qs[tt * DMAX + d], sq);
-        sk = fmaf(ks[tt * DMAX + d], ks[tt * DMAX + d], sk);
-      }
-      sq = wave_sum(sq);
-      sk = wave_sum(sk);
-      const float iq = q_scale / sqrtf(sq + 1e-6f), ik = 1.0f / sqrtf(sk + 1e-6f);
-      for (int d = lane; d < DMAX; d += 64) {
-        qs[tt * DMAX + d] *= iq;
-        ks[tt * DMAX + d] *= ik;
-      }
+    if (wide && c0 + GRP < t1) fetch(c0 + GRP, min(GRP, t1 - c0 - GRP));
+    // unit vectors: 16 lanes a row of q or k, their sum of squares joined inside the lanes' row
+    for (int item = tid >> 4; item < 2 * n; item += nt >> 4) {
+      float* row = ((item & 1) ? ks : qs) + (item >> 1) * DMAX;
+      const int l16 = tid & 15;
+      float ss = 0.f;
+      for (int d = l16; d < DMAX; d += 16) ss = fmaf(row[d], row[d], ss);
+      ss = sum16(ss);
+      const float inv = ((item & 1) ? 1.0f : q_scale) / sqrtf(ss + 1e-6f);
+      for (int d = l16; d < DMAX; d += 16) row[d] *= inv;
     }
     __syncthreads();
     // the walk: no barrier, three lane permutations a sum.  What the next token needs first (its k, v,
@@ -118,7 +197,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
     {
       const float4* k4 = (const float4*)ks + j;
 #pragma unroll
-      for (int i = 0; i < CH; i++) kn[i] = k4[8 * i];
+      for (int i = 0; i < CH; i++) kn[i] = k4[DS * i];
       vn = ov[col];
       bn = beta[0];
       gn = dec[0];
@@ -130,12 +209,12 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
 #pragma unroll
       for (int i = 0; i < CH; i++) {
         kk[i] = kn[i];
-        qq[i] = q4[8 * i];
+        qq[i] = q4[DS * i];
       }
       if (tt + 1 < n) {
         const float4* k4 = (const float4*)(ks + (tt + 1) * DMAX) + j;
 #pragma unroll
-        for (int i = 0; i < CH; i++) kn[i] = k4[8 * i];
+        for (int i = 0; i < CH; i++) kn[i] = k4[DS * i];
         vn = ov[(tt + 1) * COLS + col];
         bn = beta[tt + 1];
         gn = dec[tt + 1];
@@ -152,7 +231,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
         a2 = fmaf(s[4 * i + 2], kk[i].z, a2);
         a3 = fmaf(s[4 * i + 3], kk[i].w, a3);
       }
-      const float dot = sum8((a0 + a1) + (a2 + a3));
+      const float dot = DS == 16 ? sum16((a0 + a1) + (a2 + a3)) : sum8((a0 + a1) + (a2 + a3));
       const float u = bt * (vt - dot);
       a0 = a1 = a2 = a3 = 0.f;
 #pragma unroll
@@ -166,7 +245,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
         a2 = fmaf(s[4 * i + 2], qq[i].z, a2);
         a3 = fmaf(s[4 * i + 3], qq[i].w, a3);
       }
-      const float o = sum8((a0 + a1) + (a2 + a3));
+      const float o = DS == 16 ? sum16((a0 + a1) + (a2 + a3)) : sum8((a0 + a1) + (a2 + a3));
       // a column's v of this token was read (by its eight lanes, all in one wave) before the
       // read-out takes its place
       if (j == 0) ov[tt * COLS + col] = o;
@@ -197,7 +276,7 @@ __global__ __launch_bounds__(1024) void delta_rule_kernel(
     for (int i = 0; i < CH; i++)
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        const int d = 4 * (j + 8 * i) + c;
+        const int d = 4 * (j + DS * i) + c;
         if (d < D) S[(size_t)d * E + e] = s[4 * i + c];
       }
   }
@@ -246,22 +325,41 @@ int zk_delta_rule(const void* qkv, int ld, int k_off, int v_off, const void* z, 
   const bool scratch = raw != nullptr && positions != nullptr;
   ZK_REQUIRE(E <= DELTA_COLS || scratch, "zk_delta_rule: heads of more than 128 value channels need scratch");
   if (R == 0 || T == 0) return 0;
-  const int per_block = (scratch && max_q_len > DELTA_GROUP && E > DELTA_COLS_LONG) ? DELTA_COLS_LONG : DELTA_COLS;
+  const int DMAX = D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+  // long portions: 16 lanes a column and 16 columns a block, so that a token costs a lane fewer steps
+  // and a head spreads over more compute units; the heads' norm then follows in a kernel of its own
+  const bool spread = scratch && max_q_len > DELTA_GROUP && E > DELTA_COLS_LONG && DMAX >= 64;
+  // (a head of more than 128 rows always has 16 lanes a column: eight would hold more rows each than registers)
+  const int DS = (spread || DMAX == 256) ? 16 : 8;
+  const int per_block = spread ? DELTA_COLS_LONG : DS == 16 ? DELTA_COLS / 2 : DELTA_COLS;
+  ZK_REQUIRE(E <= per_block || scratch, "zk_delta_rule: a head that spans several blocks needs scratch");
   const int blocks_e = (E + per_block - 1) / per_block;
-  const int cols = E < per_block ? (E + 7) / 8 * 8 : per_block;         // whole waves: 8 columns each
-  const int threads = cols * 8;
-  const int RD = D <= 32 ? 4 : D <= 64 ? 8 : D <= 128 ? 16 : 32;
-  const size_t lds = ((size_t)DELTA_GROUP * (2 * 8 * RD + cols) + 2 * DELTA_GROUP) * sizeof(float);
+  const int unit = 64 / DS;                                             // columns of a wave
+  const int cols = E < per_block ? (E + unit - 1) / unit * unit : per_block;
+  const int threads = cols * DS;
+  const int GRP = (spread && DMAX <= 128) ? 2 * DELTA_GROUP : DELTA_GROUP;
+  const size_t lds = ((size_t)GRP * (2 * DMAX + cols) + 2 * GRP) * sizeof(float);
+  // rows in whole groups of eight values at addresses that are whole groups too, and few enough of them a thread
+  const int wide = (D % 8 == 0 && E % 8 == 0 && cols % 8 == 0 && ld % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 &&
+                    (uintptr_t)qkv % 32 == 0 && 2 * GRP * (D / 8) <= (spread ? 4 : 1) * threads && GRP * (cols / 8) <= threads &&
+                    GRP <= threads) ? 1 : 0;
   dim3 grid(R, H, blocks_e);
   float* raw_arg = blocks_e > 1 ? raw : nullptr;
-#define LAUNCH(N)                                                                                                     \
-  delta_rule_kernel<N><<<grid, threads, lds, (hipStream_t)stream>>>(                                                  \
+#define LAUNCH(C, L, P)                                                                                               \
+  delta_rule_kernel<C, L, P><<<grid, threads, lds, (hipStream_t)stream>>>(                                             \
       (const act_t*)qkv, ld, k_off, v_off, (const act_t*)z, ldz, ba, A_log, dt_bias, gain, state, slot_words,         \
-      offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, G, D, E, eps, cols)
-  if (RD == 4) LAUNCH(4);
-  else if (RD == 8) LAUNCH(8);
-  else if (RD == 16) LAUNCH(16);
-  else LAUNCH(32);
+      offset_words, q_start, slot_of_req, (act_t*)out, raw_arg, H, G, D, E, eps, cols, GRP, wide)
+  if (spread) {                                    // 16 lanes a column, blocks of 256 threads
+    if (DMAX == 64) LAUNCH(1, 16, 4);
+    else if (DMAX == 128) LAUNCH(2, 16, 4);
+    else LAUNCH(4, 16, 4);
+  } else if (DS == 8) {
+    if (DMAX == 32) LAUNCH(1, 8, 1);
+    else if (DMAX == 64) LAUNCH(2, 8, 1);
+    else LAUNCH(4, 8, 1);
+  } else {
+    LAUNCH(4, 16, 1);
+  }
 #undef LAUNCH
   if (blocks_e > 1) {
     dim3 fg(T, H);

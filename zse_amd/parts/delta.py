@@ -88,7 +88,7 @@ class DeltaRule(Part):
         out = ctx.alloc((T, self.vv))
         z_ptr = qkvz.ptr + (2 * self.qk + self.vv) * (4 if ctx.dtype == F32 else 2)
         # read-outs before their norm, for steps in which a head's value channels spread over several blocks
-        raw = ctx.alloc((T, self.vv), F32) if (E > 128 or ctx.max_q_len > 16) else None
+        raw = ctx.alloc((T, self.vv), F32) if (E > 64 or ctx.max_q_len > 16) else None
         k.zk_delta_rule(qkv.ptr, 2 * self.qk + self.vv, self.qk, 2 * self.qk, z_ptr, ld, ba.ptr, self.A_log.ptr,
                         self.dt_bias.ptr, self.gain.ptr, ctx.state.ptr, ctx.state.shape[1], cache.state_offset // 4,
                         ctx.q_start, ctx.slot_of_req, ctx.positions, out.ptr, raw.ptr if raw is not None else None, T,
