@@ -79,6 +79,18 @@ __device__ __forceinline__ void load8(const __bf16* p, float v[8]) {
   for (int i = 0; i < 8; i++) v[i] = (float)t[i];
 }
 
+// A wave's sum with the steps inside a row of 16 lanes done by lane permutations of the vector unit
+// (lane i with 15 - i, with 7 - i, inside the quads), the two steps across rows through local memory.
+__device__ __forceinline__ float wave_sum_rows(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x140, 0xf, 0xf, false));   // row_mirror
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x141, 0xf, 0xf, false));   // row_half_mirror
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0xB1, 0xf, 0xf, false));    // quad_perm [1,0,3,2]
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x4E, 0xf, 0xf, false));    // quad_perm [2,3,0,1]
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
 // The dot product of a weight row and a row in local memory, over a wave; the same order of sums
 // whatever the step (eight channels a lane in turn where rows are whole groups of eight).
 __device__ __forceinline__ float row_dot(const act_t* __restrict__ w, const float* __restrict__ x, int n, int lane) {
@@ -93,7 +105,7 @@ __device__ __forceinline__ float row_dot(const act_t* __restrict__ w, const floa
   } else {
     for (int i = lane; i < n; i += 64) a = fmaf(to_f32(w[i]), x[i], a);
   }
-  return wave_sum(a);
+  return wave_sum_rows(a);
 }
 
 // ---- few tokens: y[(t, k), n] = act(Wg[e] x', Wu[e] x'), a wave per row pair
