@@ -230,6 +230,26 @@ def test_experts_grouped_on_the_matrix_cores(T, E, top, W, F):
     assert np.abs(grouped - rows).max() < 0.01 * big          # a bfloat16 rounding of y apart at most
 
 
+@pytest.mark.parametrize("M", [3, 16, 40, 200])
+def test_the_clamped_gate_in_the_products_epilogue(M):
+    """act(x Wg^T, x Wu^T) straight from the matrix-core product's float sums, for every kernel the
+    number of rows picks; the clamps bite on both sides."""
+    from zse_amd.runtime.device import Runtime
+    rt = Runtime.get()
+    k = rt.kernels("bfloat16")
+    rng = np.random.default_rng(M)
+    K, F, limit = 96, 80, 1.25
+    x = bf16(rng.normal(size=(M, K)))
+    w = bf16(rng.normal(0, 2.5 / np.sqrt(K), (2 * F, K)))
+    g, u = x.astype(np.float64) @ w[:F].T, x.astype(np.float64) @ w[F:].T
+    assert (g > limit).mean() > 0.05 and (np.abs(u) > limit).mean() > 0.1
+    g, u = np.minimum(g, limit), np.clip(u, -limit, limit)
+    want = g * P.sigmoid(1.702 * g) * (u + 1.0)
+    out = rt.empty((M, F), "bfloat16")
+    k.zk_gemm_bf16(up16(rt, x).ptr, K, up16(rt, w).ptr, out.ptr, F, 0, M, F, K, 6, limit, 0, None, 0, None, rt.stream)
+    assert np.abs(rt.download_f32(out) - want).max() < 0.02 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("kn", [1, 0])
 def test_products_per_head(dev, kn):
     rt, k = dev

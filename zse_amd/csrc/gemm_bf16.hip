@@ -53,7 +53,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // <= 0: none) and that value's column in ``partials`` [M][strips] as (float, int), larger value
 // first, equal values to the lower column, NaN never, which a joining kernel reduces to one
 // column a row: the greedy choice without the logits ever reaching memory.
-enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4, EPI_RELU = 5 };
+enum { EPI_NONE = 0, EPI_SOFTCAP = 1, EPI_GELU_TANH = 2, EPI_SILU = 3, EPI_PICK = 4, EPI_RELU = 5, EPI_CLAMPED = 6 };
 
 struct Pick {
   float value;
@@ -95,8 +95,14 @@ __device__ __forceinline__ float epi_gelu_tanh(float g) {
   const float u = k * (g + 0.044715f * g * g * g);
   return g * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
 }
-__device__ __forceinline__ float epi_gate(float g, float u, int epi) {
+// cap: the limit of the clamped gate (g = min(g, cap), u = clamp(u, -cap, cap): g sigmoid(1.702 g) (u + 1))
+__device__ __forceinline__ float epi_gate(float g, float u, int epi, float cap) {
   if (epi == EPI_RELU) return fmaxf(g, 0.f) * u;
+  if (epi == EPI_CLAMPED) {
+    g = fminf(g, cap);
+    u = fminf(fmaxf(u, -cap), cap);
+    return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+  }
   return (epi == EPI_GELU_TANH ? epi_gelu_tanh(g) : g / (1.0f + expf(-g))) * u;
 }
 
@@ -375,7 +381,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const __bf16* __re
       const int n = n0 + 4 * kq + i;
       if (n >= N) continue;
       float x = v[0][i];
-      if (GATED) x = epi_gate(x, v[NS - 1][i], epi);
+      if (GATED) x = epi_gate(x, v[NS - 1][i], epi, cap);
       else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
       if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
       else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
@@ -415,7 +421,7 @@ __device__ __forceinline__ void tile_store_quad(const f32x4& x0, const f32x4& x1
     if (GATED) {
       const int n = n0 + wn * 32 + c;
       if (n < N) {
-        const float x = epi_gate(x0[e], x1[e], epi);
+        const float x = epi_gate(x0[e], x1[e], epi, cap);
         if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
         else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
       }
@@ -465,7 +471,7 @@ __device__ __forceinline__ void tile_store_staged(const f32x16 (&acc)[WMT][2], _
       for (int e = 0; e < 4; e++) {
         x[e] = acc[i][0][4 * b + e];
         y[e] = acc[i][1][4 * b + e];
-        if (GATED) x[e] = epi_gate(x[e], y[e], epi);
+        if (GATED) x[e] = epi_gate(x[e], y[e], epi, cap);
         else if (epi == EPI_SOFTCAP) {
           x[e] = cap * tanhf(x[e] / cap);
           y[e] = cap * tanhf(y[e] / cap);
@@ -984,7 +990,7 @@ __device__ __forceinline__ void mid_store(const f32x4 (&acc)[GATED ? 2 : 1][MT],
       const int n = strip * 16 + 4 * kq + i;
       if (n >= N) continue;
       float x = acc[0][mt][i];
-      if (GATED) x = epi_gate(x, acc[GATED ? 1 : 0][mt][i], epi);
+      if (GATED) x = epi_gate(x, acc[GATED ? 1 : 0][mt][i], epi, cap);
       else if (epi == EPI_SOFTCAP) x = cap * tanhf(x / cap);
       if (c_is_f32) ((float*)C)[(size_t)m * ldc + n] = x;
       else ((__bf16*)C)[(size_t)m * ldc + n] = (__bf16)x;
@@ -1155,7 +1161,7 @@ __global__ __launch_bounds__(256) void gemm_join_kernel(const float* __restrict_
   for (int i = 0; i < 4; i++) {
     if (n + i >= N) continue;
     float v = x[i];
-    if (GATED) v = epi_gate(v, y[i], epi);
+    if (GATED) v = epi_gate(v, y[i], epi, cap);
     else if (epi == EPI_SOFTCAP) v = cap * tanhf(v / cap);
     if (c_is_f32) ((float*)C)[(size_t)m * ldc + n + i] = v;
     else ((__bf16*)C)[(size_t)m * ldc + n + i] = (__bf16)v;
@@ -1354,7 +1360,7 @@ extern "C" int zk_strip_layout(const void* src, void* dst, int N, int K, void* s
   return zk_launch_status("zk_strip_layout");
 }
 
-// epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate, 5 relu gate.  For the gated
+// epi: 0 none, 1 soft cap (cap > 0), 2 gelu_tanh gate, 3 silu gate, 5 relu gate, 6 clamped gate (cap: its limit).  For the gated
 // epilogues W is [2N, K] (gate rows, then up rows) and C is [M, N].
 // w_strip: W is in strip layout (zk_strip_layout), which needs K % 32 == 0 and, for the
 // gated epilogues, N % 16 == 0.
@@ -1423,10 +1429,10 @@ static int gemm_bf16_run(const void* A, int lda, const void* W, void* C, int ldc
   ZK_REQUIRE(M >= 0 && N > 0 && K > 0, "zk_gemm_bf16: bad sizes");
   ZK_REQUIRE(K % 8 == 0 && lda % 8 == 0, "zk_gemm_bf16: K and lda must be multiples of 8");
   ZK_REQUIRE(lda >= K && ldc >= N, "zk_gemm_bf16: leading dimensions too small");
-  ZK_REQUIRE(epi >= 0 && epi <= EPI_RELU, "zk_gemm_bf16: unknown epilogue");
-  ZK_REQUIRE(epi != EPI_SOFTCAP || cap > 0.f, "zk_gemm_bf16: soft cap must be positive");
+  ZK_REQUIRE(epi >= 0 && epi <= EPI_CLAMPED, "zk_gemm_bf16: unknown epilogue");
+  ZK_REQUIRE((epi != EPI_SOFTCAP && epi != EPI_CLAMPED) || cap > 0.f, "zk_gemm_bf16: soft cap or clamp limit must be positive");
   ZK_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "zk_gemm_bf16: operands must be 16-byte aligned");
-  const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU || epi == EPI_RELU;
+  const bool gated = epi == EPI_GELU_TANH || epi == EPI_SILU || epi == EPI_RELU || epi == EPI_CLAMPED;
   ZK_REQUIRE(!w_strip || (K % 32 == 0 && (!gated || N % 16 == 0)), "zk_gemm_bf16: strip layout needs K % 32 == 0 (and N % 16 == 0 when gated)");
   if (parts) *parts = 0;
   if (M == 0) return 0;

@@ -50,6 +50,10 @@ class GatedMLP(Part):
         s = self.spec
         T, I = x.shape[0], s.intermediate_size
         last = None if out is not None else self
+        if s.activation == CLAMPED and tuned_gemm(ctx, s.hidden_size):
+            # the activation in the product's epilogue, on the float sums
+            a = linear(ctx, x, self.w_gu, ctx.alloc((T, I)), epilogue=CLAMPED, cap=float(s.limit))
+            return linear(ctx, a, self.w_down, out if out is not None else ctx.alloc((T, s.hidden_size)), last_of=last)
         if s.activation == CLAMPED:
             gu = linear(ctx, x, self.w_gu, ctx.alloc((T, 2 * I)))
             a = ctx.alloc((T, I))

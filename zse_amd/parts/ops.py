@@ -6,7 +6,8 @@ import ctypes
 from ..runtime.device import BF16, F32, Tensor
 
 
-EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3, "relu": 5}
+EPILOGUES = {None: 0, "softcap": 1, "gelu_tanh": 2, "silu": 3, "relu": 5, "clamped_swiglu": 6}
+GATED = ("gelu_tanh", "silu", "relu", "clamped_swiglu")
 
 
 def tuned_gemm(ctx, K: int) -> bool:
@@ -23,7 +24,8 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     library only the plain product exists; the bf16 library picks a matrix-core
     kernel by the number of rows.  ``epilogue`` (matrix-core product only):
     "softcap" applies cap * tanh(x / cap); "gelu_tanh" / "silu" / "relu" take w as
-    [2N, K], gate rows first, and store act(gate) * up.
+    [2N, K], gate rows first, and store act(gate) * up; "clamped_swiglu" likewise, with ``cap`` as
+    its limit: g = min(gate, cap), u = clamp(up, -cap, cap), g sigmoid(1.702 g) (u + 1).
 
     ``last_of``: the part whose result this product is (it passes itself).  When the block
     that called that very part has said that partial sums are welcome (``ctx.sums_welcome`` is
@@ -35,7 +37,7 @@ def linear(ctx, x: Tensor, w: Tensor, out: Tensor, epilogue=None, cap: float = 0
     such a tensor itself, whoever called it.
     """
     M, K = x.shape
-    gated = epilogue in ("gelu_tanh", "silu", "relu")
+    gated = epilogue in GATED
     N, K2 = w.shape
     if gated:
         N //= 2
